@@ -1,0 +1,36 @@
+"""Build the CPU oracle (test infrastructure) with gcc.
+
+  libbcpnn_oracle.so       strict IEEE restatement (the checker)
+  libbcpnn_oracle_fast.so  the reference's flag set (CMakeLists.txt:18-24,39-40), timed as the CPU baseline
+
+-march=x86-64-v3 stands in for the reference's -march=native so that a library built on one host
+still runs on another.
+
+The reference's own kernels_openmp_internal.cc is NOT built: it includes <cblas.h>, which this image
+does not provide, and writing a substitute header is not a reference build.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SRC = os.path.join(HERE, "bcpnn_oracle.c")
+
+VARIANTS = {
+    "libbcpnn_oracle.so": ["-O2", "-ffp-contract=off", "-fopenmp"],
+    "libbcpnn_oracle_fast.so": ["-O3", "-march=x86-64-v3", "-ffast-math", "-fopenmp"],
+}
+
+
+def build(verbose=False):
+    for name, flags in VARIANTS.items():
+        cmd = ["gcc", "-std=c11", "-fPIC", "-shared", "-Wall", "-Wextra", *flags, "-o",
+               os.path.join(HERE, name), SRC, "-lm"]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.run(cmd, check=True, cwd=HERE)
+
+
+if __name__ == "__main__":
+    build(verbose=True)
+    sys.exit(0)
