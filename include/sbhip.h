@@ -1,0 +1,197 @@
+/*
+ * sbhip.h -- C ABI of libsbhip.so, the MI355X (gfx950) backend of the BCPNN layer training and
+ * inference step.
+ *
+ * Conventions
+ *   - plain C types only; every function returns 0 on success or a negative sb_status, never
+ *     exits the process (the reference's CUDA path calls exit() on error,
+ *     BCPNN/backend/full_cuda_backend/helpers_cuda.h:7-27); sb_last_error() gives the message.
+ *   - "d_" pointers are device (HBM) pointers, "h_" pointers are host pointers.
+ *   - all matrices are dense row-major: x[B,N], y[B,M], W[N,M], Cij[N,M], wmask[N,H] (uint8).
+ *     N = in_features, H = hypercolumns, Mc = minicolumns, M = H*Mc, B = batch rows.
+ *   - every launch goes to one library-owned stream, in call order; calls return without waiting
+ *     for the GPU unless stated.  A handle must not be used from two threads at once.
+ *   - the _f32 / _f64 suffix is the element type of every real-valued array of that call.
+ *
+ * The per-kernel entry points carry the names of the reference's kernel module
+ * (BCPNN/backend/_kernels/kernels_openmp_internal.cc:460-478); the sb_net_* entry points are what a
+ * pybind11 backend object of the shape of PyNetwork<REAL>
+ * (BCPNN/backend/full_cuda_backend/backend_full_cuda_internals.cu:648-781) binds.
+ */
+#ifndef SBHIP_H
+#define SBHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum sb_status {
+  SB_OK = 0,
+  SB_ERR_INVALID = -1,   /* bad argument: null pointer, non-positive size, h >= H, ... */
+  SB_ERR_HIP = -2,       /* a HIP runtime call failed */
+  SB_ERR_STATE = -3,     /* call order: no dataset, unknown layer, not initialised */
+  SB_ERR_UNSUPPORTED = -4
+} sb_status;
+
+typedef enum sb_dtype { SB_F32 = 0, SB_F64 = 1 } sb_dtype;
+
+/* ---- library ---------------------------------------------------------------------------------
+ * sb_init replaces the module-level initialize() of the reference's GPU backend
+ * (backend_full_cuda_internals.cu:757-762): selects the device and creates the stream. */
+int sb_init(int device);
+int sb_shutdown(void);
+const char *sb_last_error(void);
+int sb_abi_version(void);
+/* Blocks until everything enqueued so far has finished. */
+int sb_sync(void);
+/* The library's stream as a hipStream_t, for callers that time or order work with HIP events. */
+void *sb_stream(void);
+
+/* ---- device memory for callers that have no HIP runtime of their own (ctypes tests, bench) --- */
+int sb_malloc(void **d_ptr, size_t bytes);
+int sb_free(void *d_ptr);
+int sb_memcpy_h2d(void *d_dst, const void *h_src, size_t bytes); /* synchronous */
+int sb_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes); /* synchronous */
+int sb_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes); /* stream-ordered */
+int sb_fill_bytes(void *d_dst, int value, size_t bytes);         /* stream-ordered fill kernel */
+
+/* ---- per-kernel entry points (device pointers) ------------------------------------------------ */
+
+/* act[B,M] = x[B,N] . W[N,M] + bias[M]   (act is overwritten)
+ * replaces update_state_float32/64 -> matmul_add_bias, kernels_openmp_internal.cc:70-87,342-358 */
+int sb_update_state_f32(float *d_act, const float *d_x, const float *d_W, const float *d_bias,
+                        long B, long N, long M);
+int sb_update_state_f64(double *d_act, const double *d_x, const double *d_W, const double *d_bias,
+                        long B, long N, long M);
+
+/* in place: softmax over the Mc minicolumns of each of the H hypercolumns of each row
+ * replaces softmax_minicolumns, kernels_numpy.py:13-25 (bound by cpu_backend.py:10,24) */
+int sb_softmax_minicolumns_f32(float *d_act, long B, long H, long Mc);
+int sb_softmax_minicolumns_f64(double *d_act, long B, long H, long Mc);
+
+/* update_state followed by softmax_minicolumns in one launch (layer.compute_activation,
+ * _cpu_base_backend.py:44-51,126-133) */
+int sb_compute_activation_f32(float *d_act, const float *d_x, const float *d_W,
+                              const float *d_bias, long B, long N, long H, long Mc);
+int sb_compute_activation_f64(double *d_act, const double *d_x, const double *d_W,
+                              const double *d_bias, long B, long N, long H, long Mc);
+
+/* Ci, Cj, Cij moving averages (clamped at 0) and W = log(max(Cij,cthr^4)/(Ci*Cj)) with rows
+ * Ci<cthr and columns Cj<cthr zeroed; all in place; W is the unmasked weight.
+ * replaces update_weights_float32/64 -> vectorized_updateWeights,
+ * kernels_openmp_internal.cc:89-205,361-383 */
+int sb_update_weights_f32(float *d_Ci, float *d_Cj, float *d_Cij, const float *d_a_i,
+                          const float *d_a_o, float taupdt, float *d_W, float cthr, long B, long N,
+                          long M);
+int sb_update_weights_f64(double *d_Ci, double *d_Cj, double *d_Cij, const double *d_a_i,
+                          const double *d_a_o, double taupdt, double *d_W, double cthr, long B,
+                          long N, long M);
+
+/* replaces update_bias_float32/64, kernels_openmp_internal.cc:207-220,386-396 */
+int sb_update_bias_f32(float *d_bias, const float *d_Cj, float cthr, long M);
+int sb_update_bias_f64(double *d_bias, const double *d_Cj, double cthr, long M);
+
+/* replaces update_bias_regularized_float32/64, kernels_openmp_internal.cc:222-246,399-415 */
+int sb_update_bias_regularized_f32(float *d_bias, float *d_kbi, const float *d_Cj, float cthr,
+                                   float khalf, float pmin, float taubdt, long M);
+int sb_update_bias_regularized_f64(double *d_bias, double *d_kbi, const double *d_Cj, double cthr,
+                                   double khalf, double pmin, double taubdt, long M);
+
+/* Structural-plasticity rewiring of hypercolumn h: up to `iterations` greedy swaps between the
+ * best-scoring silent row and the worst-scoring active row of wmask[:, h] (ties: highest row index).
+ * replaces update_mask_float32/64, kernels_openmp_internal.cc:248-320,418-441 */
+int sb_update_mask_f32(uint8_t *d_wmask, const float *d_W, const float *d_Ci, const float *d_Cj,
+                       const float *d_Cij, float cthr, long N, long H, long Mc, long h,
+                       long iterations);
+int sb_update_mask_f64(uint8_t *d_wmask, const double *d_W, const double *d_Ci, const double *d_Cj,
+                       const double *d_Cij, double cthr, long N, long H, long Mc, long h,
+                       long iterations);
+
+/* W[i,j] = 0 where wmask[i, j / Mc] == 0
+ * replaces apply_mask_float32/64, kernels_openmp_internal.cc:322-335,444-458 */
+int sb_apply_mask_f32(float *d_W, const uint8_t *d_wmask, long N, long H, long Mc);
+int sb_apply_mask_f64(double *d_W, const uint8_t *d_wmask, long N, long H, long Mc);
+
+/* d_pred[b] = index of the first maximum of act[b, :]  (np.argmax, _cpu_base_backend.py:239) */
+int sb_argmax_rows_f32(const float *d_act, long B, long M, int32_t *d_pred);
+int sb_argmax_rows_f64(const double *d_act, long B, long M, int32_t *d_pred);
+
+/* One structural-plasticity layer training step on device-resident state, in the order of
+ * StructuralPlasticityLayer.train_step (cpu_backend.py:29-52): traces + weights, regularised bias,
+ * [mask rewiring of hypercolumn h when h >= 0, 16 iterations], mask apply.  d_W holds the MASKED
+ * weights on return.  d_x is the layer input, d_y its activation for the same batch. */
+int sb_plastic_train_step_f32(float *d_W, float *d_bias, float *d_Ci, float *d_Cj, float *d_Cij,
+                              float *d_kbi, uint8_t *d_wmask, const float *d_x, const float *d_y,
+                              long B, long N, long H, long Mc, float taupdt, float khalf,
+                              float pmin, float taubdt, long h);
+int sb_plastic_train_step_f64(double *d_W, double *d_bias, double *d_Ci, double *d_Cj,
+                              double *d_Cij, double *d_kbi, uint8_t *d_wmask, const double *d_x,
+                              const double *d_y, long B, long N, long H, long Mc, double taupdt,
+                              double khalf, double pmin, double taubdt, long h);
+
+/* ---- network object ---------------------------------------------------------------------------
+ * Device-resident counterpart of Network<REAL>/PyNetwork<REAL>
+ * (backend_full_cuda_internals.cu:481-644,648-754) with the cpu backend's semantics
+ * (_cpu_base_backend.py:175-314, cpu_backend.py:7-52). */
+typedef struct sb_net sb_net;
+
+int sb_net_create(sb_net **net, int dtype /* sb_dtype */);
+int sb_net_destroy(sb_net *net);
+
+/* PyNetwork::add_dense_layer (backend_full_cuda_internals.cu:653-665): counters start at the three
+ * initial values; weights and bias start at zero until sb_net_set_layer_state is called.
+ * Returns the layer index (>= 0) or a negative sb_status. */
+int sb_net_add_dense_layer(sb_net *net, long n_inputs, long hypercolumns, long minicolumns,
+                           double taupdt, double initial_Ci, double initial_Cj,
+                           double initial_Cij);
+/* PyNetwork::add_plastic_layer (backend_full_cuda_internals.cu:667-683); note pmin before khalf. */
+int sb_net_add_plastic_layer(sb_net *net, long n_inputs, long hypercolumns, long minicolumns,
+                             double taupdt, double pmin, double khalf, double taubdt,
+                             double initial_Ci, double initial_Cj, double initial_Cij);
+
+/* State arrays of a layer, by name: "weights" [N,M], "bias" [M], "Ci" [N], "Cj" [M], "Cij" [N,M],
+ * "kbi" [M] (plastic layers) in the network dtype, and "wmask" [N,H] uint8 (plastic layers).
+ * The reference keeps these as numpy attributes of the layer (_cpu_base_backend.py:31-42,107-124);
+ * `bytes` must equal the array's size.  Both calls are synchronous. */
+int sb_net_set_layer_state(sb_net *net, int layer, const char *name, const void *h_src,
+                           size_t bytes);
+int sb_net_get_layer_state(sb_net *net, int layer, const char *name, void *h_dst, size_t bytes);
+
+/* PyNetwork::initiate_training (backend_full_cuda_internals.cu:685-709): copies the training set
+ * (network dtype, images [n_samples, n_features], one-hot labels [n_samples, n_classes]) to HBM.
+ * h_labels may be NULL when only non-final layers are trained. */
+int sb_net_set_training_data(sb_net *net, const void *h_images, const void *h_labels,
+                             long n_samples, long n_features, long n_classes);
+/* PyNetwork::training_done (backend_full_cuda_internals.cu:715-722): releases the training set. */
+int sb_net_training_done(sb_net *net);
+
+/* One epoch of Network._train_layer (_cpu_base_backend.py:254-314) for `layer`:
+ *   h_sample_perm[n_samples]  the epoch's sample order (int64), batches are consecutive slices of
+ *                             maximal_batch_size rows, the last one short;
+ *   h_hc_perm[H]              the epoch's hypercolumn order (int64) for the rewiring schedule
+ *                             (:297-302), used when epoch_index > 0; may be NULL for the last layer;
+ * the last layer trains on the labels, any other on its own activation; ends with train_finalize.
+ * When n_batches / (H + 1) is zero the reference divides by zero; here no rewiring happens.
+ * Asynchronous: returns once the epoch is enqueued. */
+int sb_net_train_epoch(sb_net *net, int layer, long maximal_batch_size,
+                       const int64_t *h_sample_perm, const int64_t *h_hc_perm, long epoch_index);
+
+/* Network.evaluate (_cpu_base_backend.py:205-245): forward through every layer, count rows whose
+ * argmax equals the label's argmax.  Synchronous.  h_pred (may be NULL) receives the predicted
+ * class per row. */
+int sb_net_evaluate(sb_net *net, const void *h_images, const void *h_labels, long n_samples,
+                    long n_features, long n_classes, long maximal_batch_size, int64_t *correct,
+                    int64_t *total, int32_t *h_pred);
+
+/* Forward of rows [0, n_rows) of host images through layers 0..last_layer; the activation of
+ * last_layer [n_rows, M_last] is copied to h_act.  Synchronous. */
+int sb_net_forward(sb_net *net, const void *h_images, long n_rows, long n_features, int last_layer,
+                   long maximal_batch_size, void *h_act);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SBHIP_H */

@@ -1,0 +1,123 @@
+// Shared device-side types for the gfx950 BCPNN kernels: per-dtype MFMA traits and small helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sb {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+// Real<T>: everything the kernels need to know about one element type.
+//   VW       elements per 16-byte vector (global loads/stores move VW elements per lane)
+//   mfma     D = A(16x4) * B(4x16) + C on one wavefront; lane l feeds A[l%16][l/16] and B[l/16][l%16]
+//   acc_row  row of the 16x16 result held in accumulator register v of a lane in lane-group q=l/16
+//            (measured on gfx950: f32 -> 4*q+v, f64 -> 4*v+q); the column is always l%16
+template <typename T>
+struct Real;
+
+template <>
+struct Real<float> {
+  static constexpr int VW = 4;
+  using vec_t = f32x4;
+  using acc_t = f32x4;
+  static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int acc_row(int q, int v) { return 4 * q + v; }
+  static __device__ __forceinline__ float log_(float x) { return logf(x); }
+  static __device__ __forceinline__ float exp_(float x) { return expf(x); }
+  // single IEEE operations: the pragma keeps the compiler from contracting them into FMAs
+  static __device__ __forceinline__ float add(float a, float b) {
+#pragma clang fp contract(off)
+    return a + b;
+  }
+  static __device__ __forceinline__ float mul(float a, float b) {
+#pragma clang fp contract(off)
+    return a * b;
+  }
+  static __device__ __forceinline__ float div(float a, float b) {
+#pragma clang fp contract(off)
+    return a / b;
+  }
+};
+
+template <>
+struct Real<double> {
+  static constexpr int VW = 2;
+  using vec_t = f64x2;
+  using acc_t = f64x4;
+  static __device__ __forceinline__ acc_t mfma(double a, double b, acc_t c) {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int acc_row(int q, int v) { return 4 * v + q; }
+  static __device__ __forceinline__ double log_(double x) { return log(x); }
+  static __device__ __forceinline__ double exp_(double x) { return exp(x); }
+  static __device__ __forceinline__ double add(double a, double b) {
+#pragma clang fp contract(off)
+    return a + b;
+  }
+  static __device__ __forceinline__ double mul(double a, double b) {
+#pragma clang fp contract(off)
+    return a * b;
+  }
+  static __device__ __forceinline__ double div(double a, double b) {
+#pragma clang fp contract(off)
+    return a / b;
+  }
+};
+
+// Loads VW consecutive elements row[col .. col+VW) into out[]; elements at or beyond `limit`, or the
+// whole vector when !row_ok, read as zero.  VEC promises 16-byte alignment of row+col and
+// limit % VW == 0, so a vector is entirely inside or entirely outside.
+template <typename T, bool VEC>
+__device__ __forceinline__ void load_vw(T (&out)[Real<T>::VW], const T *row, long col, long limit,
+                                        bool row_ok) {
+  constexpr int VW = Real<T>::VW;
+  if (VEC) {
+    typename Real<T>::vec_t v = {};
+    if (row_ok && col < limit) v = *reinterpret_cast<const typename Real<T>::vec_t *>(row + col);
+#pragma unroll
+    for (int e = 0; e < VW; e++) out[e] = v[e];
+  } else {
+#pragma unroll
+    for (int e = 0; e < VW; e++) out[e] = (row_ok && col + e < limit) ? row[col + e] : T(0);
+  }
+}
+
+template <typename T, bool VEC>
+__device__ __forceinline__ void store_vw(const T (&in)[Real<T>::VW], T *row, long col, long limit) {
+  constexpr int VW = Real<T>::VW;
+  if (VEC) {
+    if (col < limit) {
+      typename Real<T>::vec_t v;
+#pragma unroll
+      for (int e = 0; e < VW; e++) v[e] = in[e];
+      *reinterpret_cast<typename Real<T>::vec_t *>(row + col) = v;
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < VW; e++)
+      if (col + e < limit) row[col + e] = in[e];
+  }
+}
+
+// The weight of one synapse from its traces, shared by the trace/weight kernel and the rewiring
+// kernels so both see bit-identical values:  log(max(cij, cthr^4) / (ci * cj)) evaluated as
+// log(max(cij, cthr^4) * (1/ci) * (1/cj)).  rci / rcj are the reciprocals, or a negative number when
+// the row / column trace is below cthr (the weight is then zero).
+template <typename T>
+__device__ __forceinline__ T trace_reciprocal(T c, T cthr) {
+  return (c < cthr) ? T(-1) : Real<T>::div(T(1), c);
+}
+template <typename T>
+__device__ __forceinline__ T weight_from_traces(T cij, T rci, T rcj, T cthr4) {
+  const T num = cij > cthr4 ? cij : cthr4;
+  const T w = Real<T>::log_(num * rci * rcj);
+  return (rci < T(0) || rcj < T(0)) ? T(0) : w;
+}
+
+}  // namespace sb

@@ -1,0 +1,83 @@
+// Host-side launchers: shape checks, kernel-variant selection and grid computation for every kernel.
+// All launches go to the stream handed in; nothing here synchronises.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+namespace sb {
+
+// Scalars of one layer narrowed to the element type the way the reference's call boundary does it:
+// Python float64 -> REAL at the pybind call (omp.cc:362-365,400-402,419-422), cthr = taupdt/2 formed in
+// float64 first (cpu_backend.py:15,31), 1-taupdt formed in double and narrowed (omp.cc:101), cthr^4 by
+// repeated multiplication in REAL (omp.cc:102).
+template <typename T>
+struct TraceScalars {
+  T tau, omt, cthr, cthr4;
+  static TraceScalars from(T taupdt, T cthr_) {
+    TraceScalars s;
+    s.tau = taupdt;
+    s.omt = (T)(1.0 - (double)taupdt);
+    s.cthr = cthr_;
+    volatile T c2 = cthr_ * cthr_;
+    volatile T c3 = c2 * cthr_;
+    s.cthr4 = c3 * cthr_;
+    return s;
+  }
+};
+
+void set_error(const std::string &msg);
+int hip_fail(hipError_t e, const char *what, const char *file, int line);
+
+#define SB_HIP(call)                                                 \
+  do {                                                               \
+    hipError_t e_ = (call);                                          \
+    if (e_ != hipSuccess) return ::sb::hip_fail(e_, #call, __FILE__, __LINE__); \
+  } while (0)
+
+#define SB_REQUIRE(cond, msg)                         \
+  do {                                                \
+    if (!(cond)) {                                    \
+      ::sb::set_error(std::string(__func__) + ": " + (msg)); \
+      return -1;                                      \
+    }                                                 \
+  } while (0)
+
+template <typename T>
+int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias, long B, long N,
+                   long H, long Mc, bool softmax);
+template <typename T>
+int launch_softmax(hipStream_t st, T *act, long B, long H, long Mc);
+template <typename T>
+int launch_counters(hipStream_t st, const T *x, const T *y, T *Ci, T *Cj, long B, long N, long M,
+                    T taupdt, int bias_mode, T *bias, T *kbi, T cthr, T khalf, T pmin, T taubdt);
+template <typename T>
+int launch_trace_weights(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci,
+                         const T *Cj, const uint8_t *wmask, long B, long N, long H, long Mc, T taupdt,
+                         T cthr);
+template <typename T>
+int launch_update_bias(hipStream_t st, T *bias, const T *Cj, T cthr, long M);
+template <typename T>
+int launch_update_bias_regularized(hipStream_t st, T *bias, T *kbi, const T *Cj, T cthr, T khalf,
+                                   T pmin, T taubdt, long M);
+// nom / csum: scratch of N elements each.  W == nullptr: weights recomputed from the traces.
+template <typename T>
+int launch_update_mask(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, const T *Cj,
+                       const T *Cij, T cthr, long N, long H, long Mc, long h, long iterations, T *nom,
+                       int *csum);
+template <typename T>
+int launch_mask_fix_weights(hipStream_t st, T *W, const uint8_t *wmask, const T *Ci, const T *Cj,
+                            const T *Cij, T cthr, long N, long H, long Mc, long h);
+template <typename T>
+int launch_apply_mask(hipStream_t st, T *W, const uint8_t *wmask, long N, long H, long Mc);
+template <typename T>
+int launch_argmax_rows(hipStream_t st, const T *act, const T *labels, long B, long M, int32_t *pred,
+                       unsigned long long *correct);
+template <typename T>
+int launch_gather_rows(hipStream_t st, T *dst, const T *src, const int64_t *idx, long rows, long cols);
+template <typename T>
+int launch_fill(hipStream_t st, T *dst, T value, size_t n);
+int launch_fill_bytes(hipStream_t st, void *dst, int value, size_t bytes);
+
+}  // namespace sb

@@ -1,0 +1,248 @@
+// Definitions of the launchers declared in sb_launch.hpp; included once per element type by
+// sb_kernels_f32.hip / sb_kernels_f64.hip, which instantiate them explicitly.
+#pragma once
+#include "sb_kernels.hpp"
+#include "sb_launch.hpp"
+
+namespace sb {
+
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static inline long cdiv(long a, long b) { return (a + b - 1) / b; }
+
+#define SB_LAUNCH_CHECK() SB_HIP(hipGetLastError())
+
+// ------------------------------------------------------------------------------------------- forward
+template <typename T, int NG, bool FUSE>
+static int forward_variant(hipStream_t st, const ForwardArgs<T> &a, dim3 grid, bool vec) {
+  if (vec)
+    hipLaunchKernelGGL((k_forward<T, NG, FUSE, true>), grid, dim3(256), 0, st, a);
+  else
+    hipLaunchKernelGGL((k_forward<T, NG, FUSE, false>), grid, dim3(256), 0, st, a);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
+int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias, long B, long N,
+                   long H, long Mc, bool softmax) {
+  constexpr int VW = Real<T>::VW;
+  constexpr int GW = 16 * VW;
+  SB_REQUIRE(act && x && W && bias, "null pointer");
+  SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");
+  const long M = H * Mc;
+  SB_REQUIRE(M < (1L << 31) && N < (1L << 31), "dimension too large");
+  SB_REQUIRE(cdiv(B, 16) <= 65535, "batch too large for one launch");
+  ForwardArgs<T> a{act, x, W, bias, B, N, M, Mc};
+  const bool base_vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(W);
+  const long need = cdiv(Mc, GW);
+  const long max_fused = sizeof(T) == 4 ? 4 : 7;
+  if (softmax && need <= max_fused) {
+    const bool vec = base_vec && (Mc % VW == 0);
+    dim3 grid((unsigned)H, (unsigned)cdiv(B, 16));
+    if (need <= 1) return forward_variant<T, 1, true>(st, a, grid, vec);
+    if (need <= 2) return forward_variant<T, 2, true>(st, a, grid, vec);
+    if (need <= 4) return forward_variant<T, 4, true>(st, a, grid, vec);
+    if constexpr (sizeof(T) == 8) return forward_variant<T, 7, true>(st, a, grid, vec);
+  }
+  {
+    dim3 grid((unsigned)cdiv(M, 2 * GW), (unsigned)cdiv(B, 16));
+    int rc = forward_variant<T, 2, false>(st, a, grid, base_vec);
+    if (rc) return rc;
+  }
+  if (softmax) return launch_softmax<T>(st, act, B, H, Mc);
+  return 0;
+}
+
+template <typename T>
+int launch_softmax(hipStream_t st, T *act, long B, long H, long Mc) {
+  SB_REQUIRE(act, "null pointer");
+  SB_REQUIRE(B > 0 && H > 0 && Mc > 0, "sizes must be positive");
+  const long groups = B * H;
+  SB_REQUIRE(cdiv(groups, 4) < (1L << 31), "too many groups");
+  hipLaunchKernelGGL((k_softmax<T>), dim3((unsigned)cdiv(groups, 4)), dim3(256), 0, st, act, groups,
+                     Mc);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------ counters
+template <typename T>
+int launch_counters(hipStream_t st, const T *x, const T *y, T *Ci, T *Cj, long B, long N, long M,
+                    T taupdt, int bias_mode, T *bias, T *kbi, T cthr, T khalf, T pmin, T taubdt) {
+  SB_REQUIRE(x && y && Ci && Cj, "null pointer");
+  SB_REQUIRE(B > 0 && N > 0 && M > 0, "sizes must be positive");
+  SB_REQUIRE(bias_mode == 0 || (bias && kbi), "bias update needs bias and kbi");
+  CountersArgs<T> a;
+  a.x = x; a.y = y; a.Ci = Ci; a.Cj = Cj; a.B = B; a.N = N; a.M = M;
+  a.tau = taupdt; a.omt = (T)(1.0 - (double)taupdt); a.fB = (T)B;
+  a.bias_mode = bias_mode; a.bias = bias; a.kbi = kbi;
+  a.cthr = cthr; a.khalf = khalf; a.pmin = pmin; a.taubdt = taubdt;
+  hipLaunchKernelGGL((k_counters<T>), dim3((unsigned)cdiv(N + M, 256)), dim3(256), 0, st, a);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------- trace + weights
+template <typename T, int RX, int RY>
+static int trace_variant(hipStream_t st, const TraceArgs<T> &a, bool vec) {
+  constexpr int GW = 16 * Real<T>::VW;
+  dim3 grid((unsigned)cdiv(a.M, 2 * RY * GW), (unsigned)cdiv(a.N, 2 * RX * GW));
+  if (grid.y > 65535) {
+    set_error("launch_trace_weights: in_features too large for one launch");
+    return -1;
+  }
+  if (vec)
+    hipLaunchKernelGGL((k_trace_weights<T, RX, RY, true, true>), grid, dim3(256), 0, st, a);
+  else
+    hipLaunchKernelGGL((k_trace_weights<T, RX, RY, false, true>), grid, dim3(256), 0, st, a);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
+int launch_trace_weights(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci,
+                         const T *Cj, const uint8_t *wmask, long B, long N, long H, long Mc, T taupdt,
+                         T cthr) {
+  constexpr int VW = Real<T>::VW;
+  SB_REQUIRE(x && y && Cij && W && Ci && Cj, "null pointer");
+  SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");
+  const long M = H * Mc;
+  SB_REQUIRE(M < (1L << 31) && N < (1L << 31), "dimension too large");
+  const TraceScalars<T> s = TraceScalars<T>::from(taupdt, cthr);
+  TraceArgs<T> a;
+  a.x = x; a.y = y; a.Cij = Cij; a.W = W; a.Ci = Ci; a.Cj = Cj; a.wmask = wmask;
+  a.B = B; a.N = N; a.M = M; a.H = H; a.Mc = Mc;
+  a.tau = s.tau; a.omt = s.omt; a.invB = (T)1 / (T)B; a.cthr = s.cthr; a.cthr4 = s.cthr4;
+  const bool vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(y) && aligned16(Cij) &&
+                   aligned16(W);
+  if constexpr (sizeof(T) == 4)
+    return trace_variant<T, 1, 1>(st, a, vec);
+  else
+    return trace_variant<T, 1, 2>(st, a, vec);
+}
+
+// ---------------------------------------------------------------------------------------------- bias
+template <typename T>
+int launch_update_bias(hipStream_t st, T *bias, const T *Cj, T cthr, long M) {
+  SB_REQUIRE(bias && Cj, "null pointer");
+  SB_REQUIRE(M > 0, "sizes must be positive");
+  hipLaunchKernelGGL((k_update_bias<T>), dim3((unsigned)cdiv(M, 256)), dim3(256), 0, st, bias, Cj, cthr,
+                     M);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
+int launch_update_bias_regularized(hipStream_t st, T *bias, T *kbi, const T *Cj, T cthr, T khalf,
+                                   T pmin, T taubdt, long M) {
+  SB_REQUIRE(bias && kbi && Cj, "null pointer");
+  SB_REQUIRE(M > 0, "sizes must be positive");
+  hipLaunchKernelGGL((k_update_bias_regularized<T>), dim3((unsigned)cdiv(M, 256)), dim3(256), 0, st,
+                     bias, kbi, Cj, cthr, khalf, pmin, taubdt, M);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------- mask
+template <typename T>
+int launch_update_mask(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, const T *Cj,
+                       const T *Cij, T cthr, long N, long H, long Mc, long h, long iterations, T *nom,
+                       int *csum) {
+  SB_REQUIRE(wmask && Ci && Cj && Cij && nom && csum, "null pointer");
+  SB_REQUIRE(N > 0 && H > 0 && Mc > 0, "sizes must be positive");
+  SB_REQUIRE(h >= 0 && h < H, "hypercolumn index out of range");
+  SB_REQUIRE(iterations >= 0, "iterations must be non-negative");
+  SB_REQUIRE(cdiv(N, 4) < (1L << 31), "in_features too large");
+  const TraceScalars<T> s = TraceScalars<T>::from(T(0), cthr);
+  MaskArgs<T> a;
+  a.wmask = wmask; a.W = W; a.Ci = Ci; a.Cj = Cj; a.Cij = Cij; a.cthr = cthr; a.cthr4 = s.cthr4;
+  a.N = N; a.M = H * Mc; a.H = H; a.Mc = Mc; a.h = h; a.iterations = iterations; a.nom = nom;
+  a.csum = csum;
+  hipLaunchKernelGGL((k_mask_scores<T>), dim3((unsigned)cdiv(N, 4)), dim3(256), 0, st, a);
+  SB_LAUNCH_CHECK();
+  if (iterations > 0) {
+    hipLaunchKernelGGL((k_mask_swap<T>), dim3(1), dim3(1024), 0, st, a);
+    SB_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+template <typename T>
+int launch_mask_fix_weights(hipStream_t st, T *W, const uint8_t *wmask, const T *Ci, const T *Cj,
+                            const T *Cij, T cthr, long N, long H, long Mc, long h) {
+  SB_REQUIRE(W && wmask && Ci && Cj && Cij, "null pointer");
+  SB_REQUIRE(h >= 0 && h < H, "hypercolumn index out of range");
+  const TraceScalars<T> s = TraceScalars<T>::from(T(0), cthr);
+  hipLaunchKernelGGL((k_mask_fix_weights<T>), dim3((unsigned)cdiv(N * Mc, 256)), dim3(256), 0, st, W,
+                     wmask, Ci, Cj, Cij, cthr, s.cthr4, N, H * Mc, H, Mc, h);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
+int launch_apply_mask(hipStream_t st, T *W, const uint8_t *wmask, long N, long H, long Mc) {
+  SB_REQUIRE(W && wmask, "null pointer");
+  SB_REQUIRE(N > 0 && H > 0 && Mc > 0, "sizes must be positive");
+  const long total = N * H * Mc;
+  const long blocks = cdiv(total, 256) < 8192 ? cdiv(total, 256) : 8192;
+  hipLaunchKernelGGL((k_apply_mask<T>), dim3((unsigned)blocks), dim3(256), 0, st, W, wmask, N, H * Mc,
+                     H, Mc);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------- classification
+template <typename T>
+int launch_argmax_rows(hipStream_t st, const T *act, const T *labels, long B, long M, int32_t *pred,
+                       unsigned long long *correct) {
+  SB_REQUIRE(act, "null pointer");
+  SB_REQUIRE(!labels || correct, "labels need a counter");
+  SB_REQUIRE(B > 0 && M > 0, "sizes must be positive");
+  hipLaunchKernelGGL((k_argmax_rows<T>), dim3((unsigned)cdiv(B, 4)), dim3(256), 0, st, act, labels, B,
+                     M, pred, correct);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
+int launch_gather_rows(hipStream_t st, T *dst, const T *src, const int64_t *idx, long rows,
+                       long cols) {
+  SB_REQUIRE(dst && src && idx, "null pointer");
+  SB_REQUIRE(rows > 0 && cols > 0 && rows < (1L << 31), "bad shape");
+  hipLaunchKernelGGL((k_gather_rows<T>), dim3((unsigned)rows), dim3(256), 0, st, dst, src, idx, rows,
+                     cols);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
+int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
+  if (n == 0) return 0;
+  SB_REQUIRE(dst, "null pointer");
+  const size_t blocks = (n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096;
+  hipLaunchKernelGGL((k_fill<T>), dim3((unsigned)blocks), dim3(256), 0, st, dst, value, n);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+#define SB_INSTANTIATE_LAUNCHERS(T)                                                                   \
+  template int launch_forward<T>(hipStream_t, T *, const T *, const T *, const T *, long, long, long, \
+                                 long, bool);                                                         \
+  template int launch_softmax<T>(hipStream_t, T *, long, long, long);                                 \
+  template int launch_counters<T>(hipStream_t, const T *, const T *, T *, T *, long, long, long, T,   \
+                                  int, T *, T *, T, T, T, T);                                         \
+  template int launch_trace_weights<T>(hipStream_t, const T *, const T *, T *, T *, const T *,        \
+                                       const T *, const uint8_t *, long, long, long, long, T, T);     \
+  template int launch_update_bias<T>(hipStream_t, T *, const T *, T, long);                           \
+  template int launch_update_bias_regularized<T>(hipStream_t, T *, T *, const T *, T, T, T, T, long); \
+  template int launch_update_mask<T>(hipStream_t, uint8_t *, const T *, const T *, const T *,         \
+                                     const T *, T, long, long, long, long, long, T *, int *);         \
+  template int launch_mask_fix_weights<T>(hipStream_t, T *, const uint8_t *, const T *, const T *,    \
+                                          const T *, T, long, long, long, long);                      \
+  template int launch_apply_mask<T>(hipStream_t, T *, const uint8_t *, long, long, long);             \
+  template int launch_argmax_rows<T>(hipStream_t, const T *, const T *, long, long, int32_t *,        \
+                                     unsigned long long *);                                           \
+  template int launch_gather_rows<T>(hipStream_t, T *, const T *, const int64_t *, long, long);       \
+  template int launch_fill<T>(hipStream_t, T *, T, size_t);
+
+}  // namespace sb

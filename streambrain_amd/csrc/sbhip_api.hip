@@ -1,0 +1,675 @@
+// C ABI of libsbhip.so (see include/sbhip.h): library context, per-kernel entry points and the
+// device-resident network object.  Host code only; kernels live in sb_kernels.hpp.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/sbhip.h"
+#include "sb_launch.hpp"
+
+namespace sb {
+
+static thread_local std::string g_error;
+void set_error(const std::string &msg) { g_error = msg; }
+int hip_fail(hipError_t e, const char *what, const char *file, int line) {
+  g_error = std::string("HIP error '") + hipGetErrorString(e) + "' from " + what + " at " + file + ":" +
+            std::to_string(line);
+  return SB_ERR_HIP;
+}
+
+struct Context {
+  bool ready = false;
+  int device = 0;
+  hipStream_t stream = nullptr;
+  // scratch of the per-kernel sb_update_mask entry point
+  void *mask_nom = nullptr;
+  int *mask_csum = nullptr;
+  long mask_cap = 0;
+};
+static Context g_ctx;
+static std::mutex g_ctx_mutex;
+
+static int require_ready() {
+  if (!g_ctx.ready) {
+    set_error("sb_init has not been called");
+    return SB_ERR_STATE;
+  }
+  return 0;
+}
+
+#define SB_READY()          \
+  do {                      \
+    int rc_ = require_ready(); \
+    if (rc_) return rc_;    \
+  } while (0)
+
+static int ensure_mask_scratch(long N) {
+  if (N <= g_ctx.mask_cap) return 0;
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  if (g_ctx.mask_nom) SB_HIP(hipFree(g_ctx.mask_nom));
+  if (g_ctx.mask_csum) SB_HIP(hipFree(g_ctx.mask_csum));
+  g_ctx.mask_nom = nullptr;
+  g_ctx.mask_csum = nullptr;
+  g_ctx.mask_cap = 0;
+  SB_HIP(hipMalloc(&g_ctx.mask_nom, (size_t)N * sizeof(double)));
+  SB_HIP(hipMalloc((void **)&g_ctx.mask_csum, (size_t)N * sizeof(int)));
+  g_ctx.mask_cap = N;
+  return 0;
+}
+
+// ======================================================================================== network
+struct Layer {
+  bool plastic = false;
+  long N = 0, H = 0, Mc = 0, M = 0;
+  double taupdt = 0, pmin = 0, khalf = 0, taubdt = 0;
+  void *W = nullptr, *bias = nullptr, *Ci = nullptr, *Cj = nullptr, *Cij = nullptr, *kbi = nullptr;
+  uint8_t *wmask = nullptr;
+  void *act = nullptr;  // [act_rows, M]
+  long act_rows = 0;
+  void *nom = nullptr;  // rewiring scratch [N]
+  int *csum = nullptr;
+};
+
+}  // namespace sb
+
+struct sb_net {
+  int dtype = SB_F32;
+  size_t esize = 4;
+  std::vector<sb::Layer> layers;
+  // training set in HBM, its per-epoch permuted copy and the permutation
+  void *X = nullptr, *Y = nullptr, *Xp = nullptr, *Yp = nullptr;
+  long Ns = 0, NF = 0, NC = 0;
+  int64_t *d_perm = nullptr;
+  int64_t *h_perm = nullptr;  // pinned staging
+  hipEvent_t perm_copied = nullptr;
+  unsigned long long *d_correct = nullptr;
+};
+
+namespace sb {
+
+static int free_dev(void *&p) {
+  if (p) SB_HIP(hipFree(p));
+  p = nullptr;
+  return 0;
+}
+
+template <typename T>
+static int layer_alloc(Layer &L, T ci0, T cj0, T cij0) {
+  hipStream_t st = g_ctx.stream;
+  const size_t nm = (size_t)L.N * L.M;
+  SB_HIP(hipMalloc(&L.W, nm * sizeof(T)));
+  SB_HIP(hipMalloc(&L.Cij, nm * sizeof(T)));
+  SB_HIP(hipMalloc(&L.bias, L.M * sizeof(T)));
+  SB_HIP(hipMalloc(&L.Cj, L.M * sizeof(T)));
+  SB_HIP(hipMalloc(&L.Ci, L.N * sizeof(T)));
+  int rc = 0;
+  if ((rc = launch_fill<T>(st, (T *)L.W, T(0), nm))) return rc;
+  if ((rc = launch_fill<T>(st, (T *)L.Cij, cij0, nm))) return rc;
+  if ((rc = launch_fill<T>(st, (T *)L.bias, T(0), L.M))) return rc;
+  if ((rc = launch_fill<T>(st, (T *)L.Cj, cj0, L.M))) return rc;
+  if ((rc = launch_fill<T>(st, (T *)L.Ci, ci0, L.N))) return rc;
+  if (L.plastic) {
+    SB_HIP(hipMalloc(&L.kbi, L.M * sizeof(T)));
+    SB_HIP(hipMalloc((void **)&L.wmask, (size_t)L.N * L.H));
+    SB_HIP(hipMalloc(&L.nom, L.N * sizeof(T)));
+    SB_HIP(hipMalloc((void **)&L.csum, L.N * sizeof(int)));
+    if ((rc = launch_fill<T>(st, (T *)L.kbi, T(1), L.M))) return rc;
+    if ((rc = launch_fill_bytes(st, L.wmask, 1, (size_t)L.N * L.H))) return rc;
+  }
+  return 0;
+}
+
+static int layer_free(Layer &L) {
+  int rc = 0;
+  void *w = L.wmask, *c = L.csum;
+  rc |= free_dev(L.W); rc |= free_dev(L.bias); rc |= free_dev(L.Ci); rc |= free_dev(L.Cj);
+  rc |= free_dev(L.Cij); rc |= free_dev(L.kbi); rc |= free_dev(w); rc |= free_dev(L.act);
+  rc |= free_dev(L.nom); rc |= free_dev(c);
+  L.wmask = nullptr; L.csum = nullptr;
+  return rc;
+}
+
+static int ensure_act(sb_net *net, long rows) {
+  for (auto &L : net->layers) {
+    if (L.act_rows >= rows) continue;
+    SB_HIP(hipStreamSynchronize(g_ctx.stream));
+    int rc = free_dev(L.act);
+    if (rc) return rc;
+    SB_HIP(hipMalloc(&L.act, (size_t)rows * L.M * net->esize));
+    L.act_rows = rows;
+  }
+  return 0;
+}
+
+template <typename T>
+static int layer_forward(const Layer &L, const T *x, long B) {
+  return launch_forward<T>(g_ctx.stream, (T *)L.act, x, (const T *)L.W, (const T *)L.bias, B, L.N, L.H,
+                           L.Mc, true);
+}
+
+// One training step of `L` on input x (and on y = its own activation or the labels), in the order of
+// cpu_backend.py:13-15 (dense) and :29-52 (plastic).  W stays masked; on rewiring steps hypercolumn h
+// is re-scored from the traces and its W columns rewritten under the new mask.
+template <typename T>
+static int layer_train_step(Layer &L, const T *x, const T *y, long B, long h) {
+  hipStream_t st = g_ctx.stream;
+  const T tau = (T)L.taupdt;
+  const T cthr = (T)(L.taupdt / 2);
+  int rc = launch_counters<T>(st, x, y, (T *)L.Ci, (T *)L.Cj, B, L.N, L.M, tau, L.plastic ? 1 : 0,
+                              (T *)L.bias, (T *)L.kbi, cthr, (T)L.khalf, (T)L.pmin, (T)L.taubdt);
+  if (rc) return rc;
+  rc = launch_trace_weights<T>(st, x, y, (T *)L.Cij, (T *)L.W, (const T *)L.Ci, (const T *)L.Cj,
+                               L.plastic ? L.wmask : nullptr, B, L.N, L.H, L.Mc, tau, cthr);
+  if (rc) return rc;
+  if (L.plastic && h >= 0) {
+    rc = launch_update_mask<T>(st, L.wmask, (const T *)nullptr, (const T *)L.Ci, (const T *)L.Cj,
+                               (const T *)L.Cij, cthr, L.N, L.H, L.Mc, h, 16, (T *)L.nom, L.csum);
+    if (rc) return rc;
+    rc = launch_mask_fix_weights<T>(st, (T *)L.W, L.wmask, (const T *)L.Ci, (const T *)L.Cj,
+                                    (const T *)L.Cij, cthr, L.N, L.H, L.Mc, h);
+    if (rc) return rc;
+  }
+  return 0;
+}
+
+template <typename T>
+static int net_train_epoch(sb_net *net, int layer, long maxB, const int64_t *h_sample_perm,
+                           const int64_t *h_hc_perm, long epoch) {
+  hipStream_t st = g_ctx.stream;
+  Layer &target = net->layers[layer];
+  const bool last = layer + 1 == (int)net->layers.size();
+  SB_REQUIRE(!last || net->Y, "the last layer trains on labels but none were given");
+  SB_REQUIRE(!last || net->NC == target.M, "label width does not match the last layer");
+  SB_REQUIRE(last || target.plastic, "a dense layer can only be trained as the last layer");
+  SB_REQUIRE(net->layers[0].N == net->NF, "image width does not match the first layer");
+  for (int l = 1; l <= layer; l++)
+    SB_REQUIRE(net->layers[l].N == net->layers[l - 1].M, "layer widths do not chain");
+  const long Ns = net->Ns;
+  for (long r = 0; r < Ns; r++)
+    SB_REQUIRE(h_sample_perm[r] >= 0 && h_sample_perm[r] < Ns, "sample index out of range");
+  int rc = ensure_act(net, maxB < Ns ? maxB : Ns);
+  if (rc) return rc;
+
+  // images[idx, :] / labels[idx, :]  (_cpu_base_backend.py:258-260)
+  if (!net->Xp) SB_HIP(hipMalloc(&net->Xp, (size_t)Ns * net->NF * net->esize));
+  if (last && !net->Yp) SB_HIP(hipMalloc(&net->Yp, (size_t)Ns * net->NC * net->esize));
+  SB_HIP(hipEventSynchronize(net->perm_copied));  // staging buffer free again
+  std::memcpy(net->h_perm, h_sample_perm, (size_t)Ns * sizeof(int64_t));
+  SB_HIP(hipMemcpyAsync(net->d_perm, net->h_perm, (size_t)Ns * sizeof(int64_t), hipMemcpyHostToDevice,
+                        st));
+  SB_HIP(hipEventRecord(net->perm_copied, st));
+  if ((rc = launch_gather_rows<T>(st, (T *)net->Xp, (const T *)net->X, net->d_perm, Ns, net->NF)))
+    return rc;
+  if (last)
+    if ((rc = launch_gather_rows<T>(st, (T *)net->Yp, (const T *)net->Y, net->d_perm, Ns, net->NC)))
+      return rc;
+
+  const long nb = (Ns + maxB - 1) / maxB;
+  const long period = nb / (target.H + 1);  // _cpu_base_backend.py:297-299
+  for (long i = 0; i < nb; i++) {
+    const long lo = i * maxB;
+    const long B = (lo + maxB <= Ns) ? maxB : Ns - lo;
+    const T *x = (const T *)net->Xp + lo * net->NF;
+    for (int l = 0; l < layer; l++) {
+      if ((rc = layer_forward<T>(net->layers[l], x, B))) return rc;
+      x = (const T *)net->layers[l].act;
+    }
+    long h = -1;
+    if (!last && epoch > 0 && period > 0 && i % period == 0) {
+      const long slot = i / period;
+      if (slot < target.H) {
+        SB_REQUIRE(h_hc_perm, "hypercolumn order missing");
+        h = h_hc_perm[slot];
+        SB_REQUIRE(h >= 0 && h < target.H, "hypercolumn index out of range");
+      }
+    }
+    if (last) {
+      // the reference also evaluates the last layer's activation here and drops it
+      // (_cpu_base_backend.py:290-295, 304-306); it has no effect on any state
+      rc = layer_train_step<T>(target, x, (const T *)net->Yp + lo * net->NC, B, -1);
+    } else {
+      if ((rc = layer_forward<T>(target, x, B))) return rc;
+      rc = layer_train_step<T>(target, x, (const T *)target.act, B, h);
+    }
+    if (rc) return rc;
+  }
+  // train_finalize, once per epoch (_cpu_base_backend.py:314; cpu_backend.py:17-18)
+  if (!target.plastic)
+    return launch_update_bias<T>(st, (T *)target.bias, (const T *)target.Cj, (T)(target.taupdt / 2),
+                                 target.M);
+  return 0;
+}
+
+template <typename T>
+static int net_forward_batches(sb_net *net, const void *h_images, const void *h_labels, long n,
+                               long NF, long NC, long maxB, int last_layer, void *h_act,
+                               int64_t *correct, int32_t *h_pred) {
+  hipStream_t st = g_ctx.stream;
+  SB_REQUIRE(!net->layers.empty(), "network has no layers");
+  SB_REQUIRE(last_layer >= 0 && last_layer < (int)net->layers.size(), "layer index out of range");
+  SB_REQUIRE(net->layers[0].N == NF, "image width does not match the first layer");
+  for (int l = 1; l <= last_layer; l++)
+    SB_REQUIRE(net->layers[l].N == net->layers[l - 1].M, "layer widths do not chain");
+  const Layer &out = net->layers[last_layer];
+  SB_REQUIRE(!h_labels || NC == out.M, "label width does not match the last layer");
+  if (n == 0) return 0;
+  int rc = ensure_act(net, maxB < n ? maxB : n);
+  if (rc) return rc;
+  // stream the set through HBM in chunks of whole batches (<= ~256 MiB of images at a time)
+  long chunk = (256L << 20) / (long)(NF * sizeof(T));
+  chunk = chunk / maxB * maxB;
+  if (chunk < maxB) chunk = maxB;
+  if (chunk > n) chunk = n;
+  void *dX = nullptr, *dY = nullptr;
+  int32_t *dP = nullptr;
+  SB_HIP(hipMalloc(&dX, (size_t)chunk * NF * sizeof(T)));
+  if (h_labels) SB_HIP(hipMalloc(&dY, (size_t)chunk * NC * sizeof(T)));
+  if (h_pred) SB_HIP(hipMalloc((void **)&dP, (size_t)chunk * sizeof(int32_t)));
+  if (h_labels) {
+    unsigned long long zero = 0;
+    SB_HIP(hipMemcpy(net->d_correct, &zero, sizeof(zero), hipMemcpyHostToDevice));
+  }
+  for (long c0 = 0; c0 < n && !rc; c0 += chunk) {
+    const long rows = (c0 + chunk <= n) ? chunk : n - c0;
+    SB_HIP(hipMemcpy(dX, (const T *)h_images + c0 * NF, (size_t)rows * NF * sizeof(T),
+                     hipMemcpyHostToDevice));
+    if (h_labels)
+      SB_HIP(hipMemcpy(dY, (const T *)h_labels + c0 * NC, (size_t)rows * NC * sizeof(T),
+                       hipMemcpyHostToDevice));
+    for (long lo = 0; lo < rows && !rc; lo += maxB) {
+      const long B = (lo + maxB <= rows) ? maxB : rows - lo;
+      const T *x = (const T *)dX + lo * NF;
+      for (int l = 0; l <= last_layer && !rc; l++) {
+        rc = layer_forward<T>(net->layers[l], x, B);
+        x = (const T *)net->layers[l].act;
+      }
+      if (rc) break;
+      if (h_labels || h_pred)
+        rc = launch_argmax_rows<T>(st, (const T *)out.act, h_labels ? (const T *)dY + lo * NC : nullptr,
+                                   B, out.M, dP ? dP + lo : nullptr, net->d_correct);
+      if (!rc && h_act)
+        SB_HIP(hipMemcpyAsync((T *)h_act + (c0 + lo) * out.M, out.act, (size_t)B * out.M * sizeof(T),
+                              hipMemcpyDeviceToHost, st));
+    }
+    if (!rc && h_pred) {
+      SB_HIP(hipMemcpyAsync(h_pred + c0, dP, (size_t)rows * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    }
+    SB_HIP(hipStreamSynchronize(st));
+  }
+  if (!rc && h_labels && correct) {
+    unsigned long long cnt = 0;
+    SB_HIP(hipMemcpy(&cnt, net->d_correct, sizeof(cnt), hipMemcpyDeviceToHost));
+    *correct = (int64_t)cnt;
+  }
+  SB_HIP(hipFree(dX));
+  if (dY) SB_HIP(hipFree(dY));
+  if (dP) SB_HIP(hipFree(dP));
+  return rc;
+}
+
+struct StateRef {
+  void *ptr;
+  size_t bytes;
+};
+
+static int layer_state(sb_net *net, int layer, const char *name, StateRef &out) {
+  SB_REQUIRE(net && name, "null pointer");
+  SB_REQUIRE(layer >= 0 && layer < (int)net->layers.size(), "layer index out of range");
+  Layer &L = net->layers[layer];
+  const size_t e = net->esize;
+  const std::string n(name);
+  if (n == "weights") out = {L.W, (size_t)L.N * L.M * e};
+  else if (n == "Cij") out = {L.Cij, (size_t)L.N * L.M * e};
+  else if (n == "bias") out = {L.bias, (size_t)L.M * e};
+  else if (n == "Cj") out = {L.Cj, (size_t)L.M * e};
+  else if (n == "Ci") out = {L.Ci, (size_t)L.N * e};
+  else if (n == "kbi" && L.plastic) out = {L.kbi, (size_t)L.M * e};
+  else if (n == "wmask" && L.plastic) out = {L.wmask, (size_t)L.N * L.H};
+  else {
+    set_error("layer_state: unknown state array '" + n + "'");
+    return SB_ERR_INVALID;
+  }
+  return 0;
+}
+
+}  // namespace sb
+
+using namespace sb;
+
+// ==================================================================================== C ABI: library
+extern "C" {
+
+int sb_abi_version(void) { return 1; }
+const char *sb_last_error(void) { return g_error.c_str(); }
+
+int sb_init(int device) {
+  std::lock_guard<std::mutex> lock(g_ctx_mutex);
+  if (g_ctx.ready) {
+    if (g_ctx.device == device) return 0;
+    set_error("sb_init: already initialised on another device");
+    return SB_ERR_STATE;
+  }
+  int count = 0;
+  SB_HIP(hipGetDeviceCount(&count));
+  SB_REQUIRE(device >= 0 && device < count, "no such device");
+  SB_HIP(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  SB_HIP(hipGetDeviceProperties(&prop, device));
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    set_error(std::string("sb_init: this library is built for gfx950 only, device is ") + prop.gcnArchName);
+    return SB_ERR_UNSUPPORTED;
+  }
+  SB_HIP(hipStreamCreate(&g_ctx.stream));
+  g_ctx.device = device;
+  g_ctx.ready = true;
+  return 0;
+}
+
+int sb_shutdown(void) {
+  std::lock_guard<std::mutex> lock(g_ctx_mutex);
+  if (!g_ctx.ready) return 0;
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  if (g_ctx.mask_nom) SB_HIP(hipFree(g_ctx.mask_nom));
+  if (g_ctx.mask_csum) SB_HIP(hipFree(g_ctx.mask_csum));
+  SB_HIP(hipStreamDestroy(g_ctx.stream));
+  g_ctx = Context();
+  return 0;
+}
+
+int sb_sync(void) {
+  SB_READY();
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  return 0;
+}
+
+void *sb_stream(void) { return g_ctx.ready ? (void *)g_ctx.stream : nullptr; }
+
+int sb_malloc(void **d_ptr, size_t bytes) {
+  SB_READY();
+  SB_REQUIRE(d_ptr, "null pointer");
+  SB_HIP(hipMalloc(d_ptr, bytes ? bytes : 1));
+  return 0;
+}
+int sb_free(void *d_ptr) {
+  SB_READY();
+  if (!d_ptr) return 0;
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  SB_HIP(hipFree(d_ptr));
+  return 0;
+}
+int sb_memcpy_h2d(void *d_dst, const void *h_src, size_t bytes) {
+  SB_READY();
+  if (!bytes) return 0;
+  SB_REQUIRE(d_dst && h_src, "null pointer");
+  SB_HIP(hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, g_ctx.stream));
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  return 0;
+}
+int sb_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes) {
+  SB_READY();
+  if (!bytes) return 0;
+  SB_REQUIRE(h_dst && d_src, "null pointer");
+  SB_HIP(hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, g_ctx.stream));
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  return 0;
+}
+int sb_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes) {
+  SB_READY();
+  if (!bytes) return 0;
+  SB_REQUIRE(d_dst && d_src, "null pointer");
+  SB_HIP(hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, g_ctx.stream));
+  return 0;
+}
+int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
+  SB_READY();
+  return launch_fill_bytes(g_ctx.stream, d_dst, value, bytes);
+}
+
+// ============================================================================ C ABI: per-kernel calls
+#define SB_DEFINE_KERNEL_API(SFX, T)                                                                   \
+  int sb_update_state_##SFX(T *act, const T *x, const T *W, const T *bias, long B, long N, long M) {   \
+    SB_READY();                                                                                        \
+    return launch_forward<T>(g_ctx.stream, act, x, W, bias, B, N, 1, M, false);                        \
+  }                                                                                                    \
+  int sb_softmax_minicolumns_##SFX(T *act, long B, long H, long Mc) {                                  \
+    SB_READY();                                                                                        \
+    return launch_softmax<T>(g_ctx.stream, act, B, H, Mc);                                             \
+  }                                                                                                    \
+  int sb_compute_activation_##SFX(T *act, const T *x, const T *W, const T *bias, long B, long N,       \
+                                  long H, long Mc) {                                                   \
+    SB_READY();                                                                                        \
+    return launch_forward<T>(g_ctx.stream, act, x, W, bias, B, N, H, Mc, true);                        \
+  }                                                                                                    \
+  int sb_update_weights_##SFX(T *Ci, T *Cj, T *Cij, const T *a_i, const T *a_o, T taupdt, T *W,        \
+                              T cthr, long B, long N, long M) {                                        \
+    SB_READY();                                                                                        \
+    int rc = launch_counters<T>(g_ctx.stream, a_i, a_o, Ci, Cj, B, N, M, taupdt, 0, nullptr, nullptr,  \
+                                cthr, T(0), T(0), T(0));                                               \
+    if (rc) return rc;                                                                                 \
+    return launch_trace_weights<T>(g_ctx.stream, a_i, a_o, Cij, W, Ci, Cj, nullptr, B, N, 1, M,        \
+                                   taupdt, cthr);                                                      \
+  }                                                                                                    \
+  int sb_update_bias_##SFX(T *bias, const T *Cj, T cthr, long M) {                                     \
+    SB_READY();                                                                                        \
+    return launch_update_bias<T>(g_ctx.stream, bias, Cj, cthr, M);                                     \
+  }                                                                                                    \
+  int sb_update_bias_regularized_##SFX(T *bias, T *kbi, const T *Cj, T cthr, T khalf, T pmin,          \
+                                       T taubdt, long M) {                                             \
+    SB_READY();                                                                                        \
+    return launch_update_bias_regularized<T>(g_ctx.stream, bias, kbi, Cj, cthr, khalf, pmin, taubdt,   \
+                                             M);                                                       \
+  }                                                                                                    \
+  int sb_update_mask_##SFX(uint8_t *wmask, const T *W, const T *Ci, const T *Cj, const T *Cij,         \
+                           T cthr, long N, long H, long Mc, long h, long iterations) {                 \
+    SB_READY();                                                                                        \
+    SB_REQUIRE(W, "null pointer");                                                                     \
+    SB_REQUIRE(N > 0, "sizes must be positive");                                                       \
+    int rc = ensure_mask_scratch(N);                                                                   \
+    if (rc) return rc;                                                                                 \
+    return launch_update_mask<T>(g_ctx.stream, wmask, W, Ci, Cj, Cij, cthr, N, H, Mc, h, iterations,   \
+                                 (T *)g_ctx.mask_nom, g_ctx.mask_csum);                                \
+  }                                                                                                    \
+  int sb_apply_mask_##SFX(T *W, const uint8_t *wmask, long N, long H, long Mc) {                       \
+    SB_READY();                                                                                        \
+    return launch_apply_mask<T>(g_ctx.stream, W, wmask, N, H, Mc);                                     \
+  }                                                                                                    \
+  int sb_argmax_rows_##SFX(const T *act, long B, long M, int32_t *pred) {                              \
+    SB_READY();                                                                                        \
+    SB_REQUIRE(pred, "null pointer");                                                                  \
+    return launch_argmax_rows<T>(g_ctx.stream, act, nullptr, B, M, pred, nullptr);                     \
+  }                                                                                                    \
+  int sb_plastic_train_step_##SFX(T *W, T *bias, T *Ci, T *Cj, T *Cij, T *kbi, uint8_t *wmask,         \
+                                  const T *x, const T *y, long B, long N, long H, long Mc, T taupdt,   \
+                                  T khalf, T pmin, T taubdt, long h) {                                 \
+    SB_READY();                                                                                        \
+    SB_REQUIRE(W && bias && Ci && Cj && Cij && kbi && wmask && x && y, "null pointer");                \
+    SB_REQUIRE(N > 0 && H > 0 && Mc > 0, "sizes must be positive");                                    \
+    SB_REQUIRE(h < H, "hypercolumn index out of range");                                               \
+    const T cthr = (T)((double)taupdt / 2);                                                            \
+    int rc = launch_counters<T>(g_ctx.stream, x, y, Ci, Cj, B, N, H * Mc, taupdt, 1, bias, kbi, cthr,  \
+                                khalf, pmin, taubdt);                                                  \
+    if (rc) return rc;                                                                                 \
+    rc = launch_trace_weights<T>(g_ctx.stream, x, y, Cij, W, Ci, Cj, wmask, B, N, H, Mc, taupdt,       \
+                                 cthr);                                                                \
+    if (rc || h < 0) return rc;                                                                        \
+    if ((rc = ensure_mask_scratch(N))) return rc;                                                      \
+    rc = launch_update_mask<T>(g_ctx.stream, wmask, (const T *)nullptr, Ci, Cj, Cij, cthr, N, H, Mc,   \
+                               h, 16, (T *)g_ctx.mask_nom, g_ctx.mask_csum);                           \
+    if (rc) return rc;                                                                                 \
+    return launch_mask_fix_weights<T>(g_ctx.stream, W, wmask, Ci, Cj, Cij, cthr, N, H, Mc, h);         \
+  }
+
+SB_DEFINE_KERNEL_API(f32, float)
+SB_DEFINE_KERNEL_API(f64, double)
+
+// ================================================================================== C ABI: network
+int sb_net_create(sb_net **net, int dtype) {
+  SB_READY();
+  SB_REQUIRE(net, "null pointer");
+  SB_REQUIRE(dtype == SB_F32 || dtype == SB_F64, "dtype must be SB_F32 or SB_F64");
+  sb_net *n = new sb_net();
+  n->dtype = dtype;
+  n->esize = dtype == SB_F32 ? 4 : 8;
+  hipError_t e = hipMalloc((void **)&n->d_correct, sizeof(unsigned long long));
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&n->perm_copied, hipEventDisableTiming);
+  if (e != hipSuccess) {
+    delete n;
+    return hip_fail(e, "sb_net_create", __FILE__, __LINE__);
+  }
+  *net = n;
+  return 0;
+}
+
+int sb_net_training_done(sb_net *net) {
+  SB_READY();
+  SB_REQUIRE(net, "null pointer");
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  int rc = 0;
+  void *p = net->d_perm;
+  rc |= free_dev(net->X); rc |= free_dev(net->Y); rc |= free_dev(net->Xp); rc |= free_dev(net->Yp);
+  rc |= free_dev(p);
+  net->d_perm = nullptr;
+  if (net->h_perm) SB_HIP(hipHostFree(net->h_perm));
+  net->h_perm = nullptr;
+  net->Ns = net->NF = net->NC = 0;
+  return rc;
+}
+
+int sb_net_destroy(sb_net *net) {
+  SB_READY();
+  if (!net) return 0;
+  int rc = sb_net_training_done(net);
+  for (auto &L : net->layers) rc |= layer_free(L);
+  if (net->d_correct) SB_HIP(hipFree(net->d_correct));
+  if (net->perm_copied) SB_HIP(hipEventDestroy(net->perm_copied));
+  delete net;
+  return rc;
+}
+
+static int add_layer(sb_net *net, bool plastic, long n_inputs, long H, long Mc, double taupdt,
+                     double pmin, double khalf, double taubdt, double ci0, double cj0, double cij0) {
+  SB_READY();
+  SB_REQUIRE(net, "null pointer");
+  SB_REQUIRE(n_inputs > 0 && H > 0 && Mc > 0, "sizes must be positive");
+  SB_REQUIRE(n_inputs < (1L << 31) && H * Mc < (1L << 31), "dimension too large");
+  Layer L;
+  L.plastic = plastic;
+  L.N = n_inputs; L.H = H; L.Mc = Mc; L.M = H * Mc;
+  L.taupdt = taupdt; L.pmin = pmin; L.khalf = khalf; L.taubdt = taubdt;
+  int rc = net->dtype == SB_F32 ? layer_alloc<float>(L, (float)ci0, (float)cj0, (float)cij0)
+                                : layer_alloc<double>(L, ci0, cj0, cij0);
+  if (rc) {
+    layer_free(L);
+    return rc;
+  }
+  net->layers.push_back(L);
+  return (int)net->layers.size() - 1;
+}
+
+int sb_net_add_dense_layer(sb_net *net, long n_inputs, long hypercolumns, long minicolumns,
+                           double taupdt, double initial_Ci, double initial_Cj, double initial_Cij) {
+  return add_layer(net, false, n_inputs, hypercolumns, minicolumns, taupdt, 0, 0, 0, initial_Ci,
+                   initial_Cj, initial_Cij);
+}
+
+int sb_net_add_plastic_layer(sb_net *net, long n_inputs, long hypercolumns, long minicolumns,
+                             double taupdt, double pmin, double khalf, double taubdt,
+                             double initial_Ci, double initial_Cj, double initial_Cij) {
+  return add_layer(net, true, n_inputs, hypercolumns, minicolumns, taupdt, pmin, khalf, taubdt,
+                   initial_Ci, initial_Cj, initial_Cij);
+}
+
+int sb_net_set_layer_state(sb_net *net, int layer, const char *name, const void *h_src, size_t bytes) {
+  SB_READY();
+  StateRef s{};
+  int rc = layer_state(net, layer, name, s);
+  if (rc) return rc;
+  SB_REQUIRE(h_src, "null pointer");
+  SB_REQUIRE(bytes == s.bytes, "size mismatch");
+  return sb_memcpy_h2d(s.ptr, h_src, bytes);
+}
+
+int sb_net_get_layer_state(sb_net *net, int layer, const char *name, void *h_dst, size_t bytes) {
+  SB_READY();
+  StateRef s{};
+  int rc = layer_state(net, layer, name, s);
+  if (rc) return rc;
+  SB_REQUIRE(h_dst, "null pointer");
+  SB_REQUIRE(bytes == s.bytes, "size mismatch");
+  return sb_memcpy_d2h(h_dst, s.ptr, bytes);
+}
+
+int sb_net_set_training_data(sb_net *net, const void *h_images, const void *h_labels, long n_samples,
+                             long n_features, long n_classes) {
+  SB_READY();
+  SB_REQUIRE(net && h_images, "null pointer");
+  SB_REQUIRE(n_samples > 0 && n_features > 0, "sizes must be positive");
+  SB_REQUIRE(!h_labels || n_classes > 0, "sizes must be positive");
+  int rc = sb_net_training_done(net);
+  if (rc) return rc;
+  const size_t xb = (size_t)n_samples * n_features * net->esize;
+  SB_HIP(hipMalloc(&net->X, xb));
+  SB_HIP(hipMemcpy(net->X, h_images, xb, hipMemcpyHostToDevice));
+  if (h_labels) {
+    const size_t yb = (size_t)n_samples * n_classes * net->esize;
+    SB_HIP(hipMalloc(&net->Y, yb));
+    SB_HIP(hipMemcpy(net->Y, h_labels, yb, hipMemcpyHostToDevice));
+  }
+  SB_HIP(hipMalloc((void **)&net->d_perm, (size_t)n_samples * sizeof(int64_t)));
+  SB_HIP(hipHostMalloc((void **)&net->h_perm, (size_t)n_samples * sizeof(int64_t), hipHostMallocDefault));
+  SB_HIP(hipEventRecord(net->perm_copied, g_ctx.stream));
+  net->Ns = n_samples;
+  net->NF = n_features;
+  net->NC = h_labels ? n_classes : 0;
+  return 0;
+}
+
+int sb_net_train_epoch(sb_net *net, int layer, long maximal_batch_size, const int64_t *h_sample_perm,
+                       const int64_t *h_hc_perm, long epoch_index) {
+  SB_READY();
+  SB_REQUIRE(net && h_sample_perm, "null pointer");
+  if (!net->X) {
+    set_error("sb_net_train_epoch: no training data (call sb_net_set_training_data)");
+    return SB_ERR_STATE;
+  }
+  SB_REQUIRE(layer >= 0 && layer < (int)net->layers.size(), "layer index out of range");
+  SB_REQUIRE(maximal_batch_size > 0, "batch size must be positive");
+  SB_REQUIRE(epoch_index >= 0, "epoch index must be non-negative");
+  return net->dtype == SB_F32
+             ? net_train_epoch<float>(net, layer, maximal_batch_size, h_sample_perm, h_hc_perm, epoch_index)
+             : net_train_epoch<double>(net, layer, maximal_batch_size, h_sample_perm, h_hc_perm,
+                                       epoch_index);
+}
+
+int sb_net_evaluate(sb_net *net, const void *h_images, const void *h_labels, long n_samples,
+                    long n_features, long n_classes, long maximal_batch_size, int64_t *correct,
+                    int64_t *total, int32_t *h_pred) {
+  SB_READY();
+  SB_REQUIRE(net && h_images && h_labels && correct && total, "null pointer");
+  SB_REQUIRE(n_samples >= 0 && n_features > 0 && n_classes > 0 && maximal_batch_size > 0, "bad sizes");
+  *correct = 0;
+  *total = n_samples;
+  const int last = (int)net->layers.size() - 1;
+  return net->dtype == SB_F32
+             ? net_forward_batches<float>(net, h_images, h_labels, n_samples, n_features, n_classes,
+                                          maximal_batch_size, last, nullptr, correct, h_pred)
+             : net_forward_batches<double>(net, h_images, h_labels, n_samples, n_features, n_classes,
+                                           maximal_batch_size, last, nullptr, correct, h_pred);
+}
+
+int sb_net_forward(sb_net *net, const void *h_images, long n_rows, long n_features, int last_layer,
+                   long maximal_batch_size, void *h_act) {
+  SB_READY();
+  SB_REQUIRE(net && h_images && h_act, "null pointer");
+  SB_REQUIRE(n_rows >= 0 && n_features > 0 && maximal_batch_size > 0, "bad sizes");
+  return net->dtype == SB_F32
+             ? net_forward_batches<float>(net, h_images, nullptr, n_rows, n_features, 0,
+                                          maximal_batch_size, last_layer, h_act, nullptr, nullptr)
+             : net_forward_batches<double>(net, h_images, nullptr, n_rows, n_features, 0,
+                                           maximal_batch_size, last_layer, h_act, nullptr, nullptr);
+}
+
+}  // extern "C"

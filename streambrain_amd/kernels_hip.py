@@ -1,0 +1,143 @@
+"""numpy-facing front end of the per-kernel C ABI entry points.
+
+Same names, argument order and return values as the reference's kernel wrapper modules
+(BCPNN/backend/_kernels/kernels_openmp.py:6-99, kernels_numpy.py:18-25): numpy arrays in, the updated
+arrays out, dispatch on float32/float64, Exception("Invalid dtype") otherwise.  Every call copies its
+operands to HBM, runs the kernel(s) through libsbhip.so and copies the results back, so this module is
+for differential testing of single kernels -- training goes through the device-resident network
+object (streambrain_amd.backend.hip_backend), which keeps all state in HBM.
+"""
+import numpy as np
+
+from . import _capi
+from ._capi import DeviceArray, check, lib, suffix
+
+
+def _dev(a, dtype=None):
+    a = np.ascontiguousarray(a if dtype is None else np.asarray(a, dtype=dtype))
+    return DeviceArray.from_numpy(a)
+
+
+def _fn(base, dtype):
+    return getattr(lib(), base + suffix(dtype))
+
+
+def _back(dst, dev):
+    """Copy a device result into the caller's array (in-place semantics of the reference)."""
+    np.copyto(dst, dev.numpy().reshape(dst.shape))
+    return dst
+
+
+def update_state(state, weights, bias, inputs):
+    dt = state.dtype
+    f = _fn("sb_update_state", dt)
+    B, N = inputs.shape
+    M = weights.shape[1]
+    assert weights.shape == (N, M) and bias.shape == (M,) and state.shape == (B, M)
+    d_act = DeviceArray((B, M), dt)
+    d_x, d_w, d_b = _dev(inputs, dt), _dev(weights, dt), _dev(bias, dt)
+    check(f(d_act.ptr, d_x.ptr, d_w.ptr, d_b.ptr, B, N, M))
+    return _back(state, d_act)
+
+
+def softmax_minicolumns(a, hypercolumns, minicolumns):
+    dt = a.dtype
+    f = _fn("sb_softmax_minicolumns", dt)
+    assert a.shape[1] == hypercolumns * minicolumns
+    d = _dev(a)
+    check(f(d.ptr, a.shape[0], hypercolumns, minicolumns))
+    return _back(a, d)
+
+
+def compute_activation(weights, bias, inputs, hypercolumns, minicolumns):
+    dt = weights.dtype
+    f = _fn("sb_compute_activation", dt)
+    B, N = inputs.shape
+    M = hypercolumns * minicolumns
+    assert weights.shape == (N, M) and bias.shape == (M,)
+    d_act = DeviceArray((B, M), dt)
+    d_x, d_w, d_b = _dev(inputs, dt), _dev(weights, dt), _dev(bias, dt)
+    check(f(d_act.ptr, d_x.ptr, d_w.ptr, d_b.ptr, B, N, hypercolumns, minicolumns))
+    return d_act.numpy()
+
+
+def update_weights(Ci, Cj, Cij, a_i, a_o, taupdt, weights, cthr):
+    dt = Ci.dtype
+    f = _fn("sb_update_weights", dt)
+    B, N = a_i.shape
+    M = a_o.shape[1]
+    assert a_o.shape[0] == B and Ci.shape == (N,) and Cj.shape == (M,)
+    assert Cij.shape == (N, M) and weights.shape == (N, M)
+    d_ci, d_cj, d_cij, d_w = _dev(Ci), _dev(Cj), _dev(Cij), _dev(weights)
+    d_x, d_y = _dev(a_i, dt), _dev(a_o, dt)
+    check(f(d_ci.ptr, d_cj.ptr, d_cij.ptr, d_x.ptr, d_y.ptr, taupdt, d_w.ptr, cthr, B, N, M))
+    return _back(Ci, d_ci), _back(Cj, d_cj), _back(Cij, d_cij), _back(weights, d_w)
+
+
+def update_bias(bias, Cj, cthr):
+    dt = bias.dtype
+    f = _fn("sb_update_bias", dt)
+    d_b, d_cj = _dev(bias), _dev(Cj, dt)
+    check(f(d_b.ptr, d_cj.ptr, cthr, bias.shape[0]))
+    return _back(bias, d_b)
+
+
+def update_bias_regularized(bias, kbi, Cj, cthr, khalf, pmin, taubdt):
+    dt = bias.dtype
+    f = _fn("sb_update_bias_regularized", dt)
+    d_b, d_k, d_cj = _dev(bias), _dev(kbi), _dev(Cj, dt)
+    check(f(d_b.ptr, d_k.ptr, d_cj.ptr, cthr, khalf, pmin, taubdt, bias.shape[0]))
+    return _back(bias, d_b), _back(kbi, d_k)
+
+
+def update_mask(wmask, weights, Ci, Cj, Cij, cthr, hypercolumns, minicolumns, h, iterations):
+    dt = weights.dtype
+    f = _fn("sb_update_mask", dt)
+    N, M = weights.shape
+    assert wmask.shape == (N, hypercolumns) and wmask.dtype == np.uint8
+    assert M == hypercolumns * minicolumns
+    d_m = _dev(wmask)
+    d_w, d_ci, d_cj, d_cij = _dev(weights), _dev(Ci, dt), _dev(Cj, dt), _dev(Cij, dt)
+    check(f(d_m.ptr, d_w.ptr, d_ci.ptr, d_cj.ptr, d_cij.ptr, cthr, N, hypercolumns, minicolumns, h,
+            iterations))
+    return _back(wmask, d_m)
+
+
+def apply_mask(weights, wmask, hypercolumns, minicolumns):
+    dt = weights.dtype
+    f = _fn("sb_apply_mask", dt)
+    N, M = weights.shape
+    assert M == hypercolumns * minicolumns
+    d_w, d_m = _dev(weights), _dev(np.asarray(wmask).astype(np.uint8))
+    check(f(d_w.ptr, d_m.ptr, N, hypercolumns, minicolumns))
+    return _back(weights, d_w)
+
+
+def argmax_rows(act):
+    dt = act.dtype
+    f = _fn("sb_argmax_rows", dt)
+    B, M = act.shape
+    d_a = _dev(act)
+    d_p = DeviceArray((B,), np.int32)
+    check(f(d_a.ptr, B, M, d_p.ptr))
+    return d_p.numpy()
+
+
+def plastic_train_step(state, inputs, outputs, hypercolumns, minicolumns, taupdt, khalf, pmin, taubdt,
+                       hypercolumn=None):
+    """One StructuralPlasticityLayer.train_step (cpu_backend.py:29-52) on a dict of numpy state arrays
+    {weights, bias, Ci, Cj, Cij, kbi, wmask}; returns the updated dict."""
+    dt = state["weights"].dtype
+    f = _fn("sb_plastic_train_step", dt)
+    B, N = inputs.shape
+    names = ("weights", "bias", "Ci", "Cj", "Cij", "kbi", "wmask")
+    dev = {k: _dev(state[k]) for k in names}
+    d_x, d_y = _dev(inputs, dt), _dev(outputs, dt)
+    check(f(*(dev[k].ptr for k in names), d_x.ptr, d_y.ptr, B, N, hypercolumns, minicolumns, taupdt,
+            khalf, pmin, taubdt, -1 if hypercolumn is None else int(hypercolumn)))
+    return {k: dev[k].numpy() for k in names}
+
+
+def sync():
+    _capi.init()
+    check(lib().sb_sync())

@@ -1,0 +1,234 @@
+"""GPU parity of every per-kernel C ABI entry point against the CPU oracle on the same seeded inputs.
+
+Tolerance (floating point): |gpu - ref| <= tol * max(|ref|, 1) with tol = 1e-5 (float32) and 1e-12
+(float64); masks, class labels and everything integer are compared bit for bit.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+DT = [np.float32, np.float64]
+TOL = {np.float32: 1e-5, np.float64: 1e-12}
+
+
+def err(a, ref):
+    a = np.asarray(a, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    return float(np.max(np.abs(a - ref) / np.maximum(np.abs(ref), 1.0))) if a.size else 0.0
+
+
+def assert_close(a, ref, dtype, what, scale=1.0):
+    e = err(a, ref)
+    assert e <= scale * TOL[dtype], f"{what}: error {e:.3e} > {scale * TOL[dtype]:.1e}"
+
+
+@pytest.fixture(scope="module")
+def k():
+    from streambrain_amd import kernels_hip
+    return kernels_hip
+
+
+SHAPES = [(1, 1, 1), (3, 5, 7), (16, 64, 64), (17, 33, 65), (128, 257, 130), (96, 1568, 300)]
+
+
+# ------------------------------------------------------------------------------------ update_state
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("B,N,M", SHAPES)
+def test_update_state(k, oracle, dtype, B, N, M):
+    rng = np.random.default_rng(B * 7 + N * 3 + M)
+    x = rng.random((B, N)).astype(dtype)
+    W = (0.1 * rng.standard_normal((N, M))).astype(dtype)
+    b = (0.1 * rng.random(M)).astype(dtype)
+    got = k.update_state(np.full((B, M), 3.0, dtype=dtype), W, b, x)
+    exact = x.astype(np.float64) @ W.astype(np.float64) + b.astype(np.float64)
+    ref = oracle.update_state(np.zeros((B, M), dtype=dtype), W, b, x)
+    # both implementations accumulate N products in REAL in different orders; each is held to the
+    # tolerance against the float64 product of the same inputs, widened by sqrt(N/64) for float32
+    scale = max(1.0, np.sqrt(N / 64.0)) if dtype == np.float32 else 4.0
+    assert_close(got, exact, dtype, "gpu vs exact", scale)
+    assert_close(ref, exact, dtype, "oracle vs exact", scale)
+
+
+# ----------------------------------------------------------------------------------------- softmax
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("B,H,Mc", [(1, 1, 1), (5, 3, 7), (128, 30, 100), (9, 2, 300), (4, 1, 10)])
+def test_softmax_minicolumns(k, oracle, dtype, B, H, Mc):
+    rng = np.random.default_rng(B + H + Mc)
+    a = (4 * rng.standard_normal((B, H * Mc))).astype(dtype)
+    got = k.softmax_minicolumns(a.copy(), H, Mc)
+    ref = oracle.softmax_minicolumns(a.copy(), H, Mc)
+    assert_close(got, ref, dtype, "softmax")
+    assert np.allclose(got.reshape(B, H, Mc).sum(2), 1.0, atol=100 * TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("B,N,H,Mc", [(1, 1, 1, 1), (7, 13, 3, 5), (128, 1568, 30, 100),
+                                      (96, 1568, 30, 100), (33, 300, 2, 200), (20, 100, 2, 256),
+                                      (16, 64, 2, 300), (40, 3000, 1, 10), (10, 50, 3, 66),
+                                      (12, 40, 2, 224)])
+def test_compute_activation_fused(k, oracle, dtype, B, N, H, Mc):
+    rng = np.random.default_rng(B + N + H + Mc)
+    M = H * Mc
+    x = rng.random((B, N)).astype(dtype)
+    W = (0.1 * rng.standard_normal((N, M))).astype(dtype)
+    b = (0.1 * rng.random(M)).astype(dtype)
+    got = k.compute_activation(W, b, x, H, Mc)
+    ref = oracle.update_state(np.zeros((B, M), dtype=dtype), W, b, x)
+    ref = oracle.softmax_minicolumns(ref, H, Mc)
+    exact = x.astype(np.float64) @ W.astype(np.float64) + b.astype(np.float64)
+    exact = np.exp(exact - exact.reshape(B, H, Mc).max(2, keepdims=True).repeat(Mc, 2).reshape(B, M))
+    exact = exact / exact.reshape(B, H, Mc).sum(2, keepdims=True).repeat(Mc, 2).reshape(B, M)
+    scale = max(1.0, np.sqrt(N / 64.0)) if dtype == np.float32 else 4.0
+    assert_close(got, exact, dtype, "gpu vs exact", scale)
+    assert_close(got, ref, dtype, "gpu vs oracle", 2 * scale)
+
+
+# -------------------------------------------------------------------------- update_weights (fused)
+def _trace_problem(rng, B, N, M, dtype):
+    x = (rng.random((B, N)) * (rng.random((B, N)) < 0.5)).astype(dtype)
+    y = rng.random((B, M)).astype(dtype)
+    Ci = (0.002 + 0.9 * rng.random(N)).astype(dtype)
+    Cj = (0.002 + 0.9 * rng.random(M)).astype(dtype)
+    Cij = (0.5 * rng.random((N, M)) * (rng.random((N, M)) < 0.9)).astype(dtype)
+    return x, y, Ci, Cj, Cij
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("B,N,M", SHAPES + [(128, 1568, 3000), (5, 130, 70), (1024, 64, 64)])
+def test_update_weights(k, oracle, dtype, B, N, M):
+    rng = np.random.default_rng(B + 2 * N + 3 * M)
+    x, y, Ci, Cj, Cij = _trace_problem(rng, B, N, M, dtype)
+    tau = 0.01
+    cthr = tau / 2  # a few Ci / Cj fall below it: zeroed rows and columns are exercised
+    W = np.full((N, M), 5.0, dtype=dtype)
+    g = k.update_weights(Ci.copy(), Cj.copy(), Cij.copy(), x, y, tau, W.copy(), cthr)
+    r = oracle.update_weights(Ci.copy(), Cj.copy(), Cij.copy(), x, y, tau, W.copy(), cthr)
+    # Ci and Cj follow the reference's summation order exactly
+    assert np.array_equal(g[0], r[0]), "Ci not bit-exact"
+    assert np.array_equal(g[1], r[1]), "Cj not bit-exact"
+    assert_close(g[2], r[2], dtype, "Cij")
+    assert_close(g[3], r[3], dtype, "W", 2.0)
+    assert np.array_equal(g[3] == 0, r[3] == 0)
+
+
+# -------------------------------------------------------------------------------------------- bias
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("M", [1, 10, 3000])
+def test_update_bias(k, oracle, dtype, M):
+    rng = np.random.default_rng(M)
+    Cj = (rng.random(M) * (rng.random(M) < 0.8)).astype(dtype)
+    got = k.update_bias(np.zeros(M, dtype=dtype), Cj, 0.01)
+    ref = oracle.update_bias(np.zeros(M, dtype=dtype), Cj, 0.01)
+    assert_close(got, ref, dtype, "bias")
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("M", [1, 10, 3000])
+def test_update_bias_regularized(k, oracle, dtype, M):
+    rng = np.random.default_rng(M + 1)
+    Cj = (rng.random(M) * (rng.random(M) < 0.8)).astype(dtype)
+    kbi = (1 + rng.standard_normal(M)).astype(dtype)
+    args = (0.0035, -139.02586632856327, 0.06195283356566607, 0.02218100432360414)
+    gb, gk = k.update_bias_regularized(np.zeros(M, dtype=dtype), kbi.copy(), Cj, *args)
+    rb, rk = oracle.update_bias_regularized(np.zeros(M, dtype=dtype), kbi.copy(), Cj, *args)
+    assert np.array_equal(gk, rk), "kbi is plain IEEE arithmetic and must be bit-exact"
+    assert_close(gb, rb, dtype, "bias")
+
+
+# -------------------------------------------------------------------------------------------- mask
+def _mask_problem(rng, N, H, Mc, dtype, density=0.1):
+    M = H * Mc
+    wmask = (rng.random((N, H)) < density).astype(np.uint8)
+    W = (0.1 * rng.standard_normal((N, M))).astype(dtype)
+    Ci = (0.05 + 0.9 * rng.random(N)).astype(dtype)
+    Cj = (0.05 + 0.9 * rng.random(M)).astype(dtype)
+    Cij = np.minimum(np.minimum(0.9 * Ci[:, None], 0.9 * Cj[None, :]), rng.random((N, M))).astype(dtype)
+    return wmask, W, Ci, Cj, Cij
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("N,H,Mc", [(1, 1, 2), (7, 2, 3), (128, 5, 20), (1568, 30, 100), (5000, 3, 4)])
+@pytest.mark.parametrize("iterations", [0, 1, 16])
+def test_update_mask_bit_exact(k, oracle, dtype, N, H, Mc, iterations):
+    rng = np.random.default_rng(N + H + Mc)
+    wmask, W, Ci, Cj, Cij = _mask_problem(rng, N, H, Mc, dtype)
+    h = int(rng.integers(0, H))
+    trace = {}
+    ref = oracle.update_mask(wmask.copy(), W, Ci, Cj, Cij, 0.01, H, Mc, h, iterations, trace=trace)
+    got = k.update_mask(wmask.copy(), W, Ci, Cj, Cij, 0.01, H, Mc, h, iterations)
+    assert np.array_equal(got, ref), f"masks differ in {(got != ref).sum()} entries, swaps {trace['swaps']}"
+    assert got[:, h].sum() == wmask[:, h].sum()
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_update_mask_ties_and_degenerate_columns(k, oracle, dtype):
+    # all scores equal: last silent row on, last active row off
+    wm = np.zeros((6, 1), dtype=np.uint8); wm[[1, 3], 0] = 1
+    Ci = np.full(6, 1e-4, dtype=dtype); Cj = np.full(3, 0.3, dtype=dtype)
+    Cij = np.full((6, 3), 1e-5, dtype=dtype); W = np.zeros((6, 3), dtype=dtype)
+    got = k.update_mask(wm.copy(), W, Ci, Cj, Cij, 0.01, 1, 3, 0, 1)
+    assert got[:, 0].tolist() == [0, 1, 0, 0, 0, 1]
+    rng = np.random.default_rng(4)
+    wmask, W, Ci, Cj, Cij = _mask_problem(rng, 40, 2, 3, dtype, density=0.4)
+    for fill in (0, 1):
+        w2 = wmask.copy(); w2[:, 1] = fill
+        assert np.array_equal(k.update_mask(w2.copy(), W, Ci, Cj, Cij, 0.01, 2, 3, 1, 16), w2)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("N,H,Mc", [(1, 1, 1), (13, 4, 5), (1568, 30, 100), (100, 7, 9)])
+def test_apply_mask(k, oracle, dtype, N, H, Mc):
+    rng = np.random.default_rng(N)
+    W = rng.standard_normal((N, H * Mc)).astype(dtype)
+    wmask = (rng.random((N, H)) < 0.5).astype(np.uint8)
+    assert np.array_equal(k.apply_mask(W.copy(), wmask, H, Mc), oracle.apply_mask(W.copy(), wmask, H, Mc))
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_argmax_rows(k, oracle, dtype):
+    rng = np.random.default_rng(0)
+    a = rng.integers(0, 4, (300, 10)).astype(dtype)  # many ties: first maximum must win
+    assert np.array_equal(k.argmax_rows(a), oracle.argmax_rows(a))
+    b = rng.standard_normal((77, 1000)).astype(dtype)
+    assert np.array_equal(k.argmax_rows(b), np.argmax(b, 1))
+
+
+# ------------------------------------------------------------------------ fused plastic train step
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("B,N,H,Mc,h", [(16, 40, 3, 8, None), (16, 40, 3, 8, 1), (128, 1568, 30, 100, None),
+                                        (128, 1568, 30, 100, 7), (96, 300, 4, 25, 3), (9, 33, 2, 7, 0)])
+def test_plastic_train_step(k, oracle, dtype, B, N, H, Mc, h):
+    import scipy.special
+    rng = np.random.default_rng(B + N + H + Mc)
+    M = H * Mc
+    tau, khalf, pmin, taubdt = 0.006908854922437549, -139.02586632856327, 0.06195283356566607, \
+        0.02218100432360414
+    x = (rng.random((B, N)) * (rng.random((B, N)) < 0.3)).astype(dtype)
+    y = scipy.special.softmax(rng.standard_normal((B, H, Mc)), axis=2).reshape(B, M).astype(dtype)
+    st = {
+        "weights": (0.1 * rng.standard_normal((N, M))).astype(dtype),
+        "bias": (0.1 * rng.random(M)).astype(dtype),
+        "Ci": (0.3 * rng.random(N)).astype(dtype),
+        "Cj": np.full(M, 1.0 / Mc, dtype=dtype),
+        "kbi": np.ones(M, dtype=dtype),
+        "wmask": (rng.random((N, H)) < 0.1).astype(np.uint8),
+    }
+    st["Cij"] = (st["Ci"][:, None] * st["Cj"][None, :] * (0.5 + rng.random((N, M)))).astype(dtype)
+    got = k.plastic_train_step(st, x, y, H, Mc, tau, khalf, pmin, taubdt, h)
+    r = {n: v.copy() for n, v in st.items()}
+    cthr = tau / 2
+    oracle.update_weights(r["Ci"], r["Cj"], r["Cij"], x, y, tau, r["weights"], cthr)
+    oracle.update_bias_regularized(r["bias"], r["kbi"], r["Cj"], cthr, khalf, pmin, taubdt)
+    if h is not None:
+        oracle.update_mask(r["wmask"], r["weights"], r["Ci"], r["Cj"], r["Cij"], cthr, H, Mc, h, 16)
+    oracle.apply_mask(r["weights"], r["wmask"], H, Mc)
+    assert np.array_equal(got["wmask"], r["wmask"])
+    if h is not None and N > 100:
+        assert not np.array_equal(r["wmask"], st["wmask"]), "the case is meant to rewire"
+    assert np.array_equal(got["Ci"], r["Ci"]) and np.array_equal(got["Cj"], r["Cj"])
+    assert np.array_equal(got["kbi"], r["kbi"])
+    assert_close(got["Cij"], r["Cij"], dtype, "Cij")
+    assert_close(got["bias"], r["bias"], dtype, "bias")
+    assert_close(got["weights"], r["weights"], dtype, "W", 2.0)
+    assert np.array_equal(got["weights"] == 0, r["weights"] == 0)
