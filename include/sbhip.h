@@ -186,6 +186,11 @@ int sb_net_evaluate(sb_net *net, const void *h_images, const void *h_labels, lon
                     long n_features, long n_classes, long maximal_batch_size, int64_t *correct,
                     int64_t *total, int32_t *h_pred);
 
+/* Predicted class (first maximal activation of the last layer, np.argmax) per row of host images;
+ * the labels-free half of Network.evaluate (_cpu_base_backend.py:235-239).  Synchronous. */
+int sb_net_predict(sb_net *net, const void *h_images, long n_samples, long n_features,
+                   long maximal_batch_size, int32_t *h_pred);
+
 /* Forward of rows [0, n_rows) of host images through layers 0..last_layer; the activation of
  * last_layer [n_rows, M_last] is copied to h_act.  Synchronous. */
 int sb_net_forward(sb_net *net, const void *h_images, long n_rows, long n_features, int last_layer,

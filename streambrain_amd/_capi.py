@@ -53,6 +53,7 @@ _PLAIN_SIGS = {
     "sb_net_train_epoch": [_P, _I, _L, _P, _P, _L],
     "sb_net_evaluate": [_P, _P, _P, _L, _L, _L, _L, ctypes.POINTER(ctypes.c_int64),
                         ctypes.POINTER(ctypes.c_int64), _P],
+    "sb_net_predict": [_P, _P, _L, _L, _L, _P],
     "sb_net_forward": [_P, _P, _L, _L, _I, _L, _P],
 }
 _RESTYPES = {"sb_last_error": ctypes.c_char_p, "sb_stream": _P}

@@ -660,6 +660,19 @@ int sb_net_evaluate(sb_net *net, const void *h_images, const void *h_labels, lon
                                            maximal_batch_size, last, nullptr, correct, h_pred);
 }
 
+int sb_net_predict(sb_net *net, const void *h_images, long n_samples, long n_features,
+                   long maximal_batch_size, int32_t *h_pred) {
+  SB_READY();
+  SB_REQUIRE(net && h_images && h_pred, "null pointer");
+  SB_REQUIRE(n_samples >= 0 && n_features > 0 && maximal_batch_size > 0, "bad sizes");
+  const int last = (int)net->layers.size() - 1;
+  return net->dtype == SB_F32
+             ? net_forward_batches<float>(net, h_images, nullptr, n_samples, n_features, 0,
+                                          maximal_batch_size, last, nullptr, nullptr, h_pred)
+             : net_forward_batches<double>(net, h_images, nullptr, n_samples, n_features, 0,
+                                           maximal_batch_size, last, nullptr, nullptr, h_pred);
+}
+
 int sb_net_forward(sb_net *net, const void *h_images, long n_rows, long n_features, int last_layer,
                    long maximal_batch_size, void *h_act) {
   SB_READY();

@@ -1,0 +1,209 @@
+"""Network-level GPU parity: the hip backend's DSL (pybind11 object over the C ABI) against the
+reference driver's recorded trajectory and against the oracle's cpu-backend restatement, on identical
+seeded inputs.  Masks and predicted labels bit-exact; floats within tol * max(|ref|, 1)."""
+import os
+
+import numpy as np
+import pytest
+
+from helpers import MNIST_HP, build_two_layer, fixture_config, one_hot_labels, rel_err, synthetic_images
+
+pytestmark = pytest.mark.gpu
+
+FIX = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "driver_trajectory_f64.npz")
+
+
+@pytest.fixture(scope="module")
+def hb():
+    from streambrain_amd.backend import hip_backend
+    return hip_backend
+
+
+def test_reference_trajectory_fixture_f64(hb):
+    g = np.load(FIX)
+    c = fixture_config(g)
+    net = build_two_layer(hb, int(c["n_in"]), int(c["H"]), int(c["Mc"]), int(c["n_out"]), c, np.float64,
+                          seed=int(c["net_seed"]))
+    l0, l1 = net._layers
+    assert np.array_equal(l0.weights, g["init_L0_weights"]) and np.array_equal(l0.wmask, g["init_L0_wmask"])
+    assert np.array_equal(l1.weights, g["init_L1_weights"]) and np.array_equal(l1.bias, g["init_L1_bias"])
+    net.fit(g["X"], g["Y"], int(c["B"]), [(0, int(c["l1_epochs"]))])
+    assert np.array_equal(l0.wmask, g["mid_L0_wmask"])
+    for name in ("weights", "bias", "Ci", "Cj", "Cij", "kbi"):
+        assert rel_err(getattr(l0, name), g[f"mid_L0_{name}"]) <= 1e-11, name
+    net.fit(g["X"], g["Y"], int(c["B"]), [(1, int(c["l2_epochs"]))])
+    for li, layer in enumerate((l0, l1)):
+        for name in ("weights", "bias", "Ci", "Cj", "Cij"):
+            assert rel_err(getattr(layer, name), g[f"final_L{li}_{name}"]) <= 1e-11, f"L{li}.{name}"
+    correct, total = net.evaluate(g["Xt"], g["Yt"], int(c["B"]))
+    assert correct.tolist() == g["correct"].tolist() and total.tolist() == g["total"].tolist()
+    assert np.array_equal(net.predict(g["Xt"], int(c["B"])), g["test_predictions"])
+    assert rel_err(net.forward(g["Xt"], int(c["B"])), g["test_activations"]) <= 1e-11
+    np.testing.assert_array_equal(np.random.rand(4), g["rng_probe_after"])
+
+
+def _run_both(hb, dtype, n_pix, H, Mc, n_out, Ns, Nt, B, e1, e2, hp, data_seed):
+    from oracle import cpu_backend as ob
+    rng = np.random.default_rng(data_seed)
+    X, Y = synthetic_images(rng, Ns, n_pix), one_hot_labels(rng, Ns, n_out)
+    Xt, Yt = synthetic_images(rng, Nt, n_pix), one_hot_labels(rng, Nt, n_out)
+    nets = []
+    for backend in (hb, ob):
+        net = build_two_layer(backend, 2 * n_pix, H, Mc, n_out, hp, dtype, seed=0)
+        net.fit(X, Y, B, [(0, e1)])
+        net.fit(X, Y, B, [(1, e2)])
+        nets.append(net)
+    return nets, (Xt, Yt)
+
+
+@pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-5), (np.float64, 1e-12)])
+def test_single_step_matches_cpu_backend(hb, dtype, tol):
+    # one batch, one epoch per layer: the north-star "after one step" bound
+    (g, r), _ = _run_both(hb, dtype, n_pix=100, H=6, Mc=20, n_out=10, Ns=64, Nt=8, B=64, e1=1, e2=1,
+                          hp=MNIST_HP, data_seed=7)
+    for li in range(2):
+        for name in ("Ci", "Cj", "Cij", "weights", "bias") + (("kbi",) if li == 0 else ()):
+            e = rel_err(getattr(g._layers[li], name), getattr(r._layers[li], name))
+            assert e <= 4 * tol, f"L{li}.{name}: {e:.3e}"
+    assert np.array_equal(g._layers[0].wmask, r._layers[0].wmask)
+
+
+def _compare_states(g, r, tol, names=("Ci", "Cj", "Cij", "weights", "bias")):
+    for li in range(2):
+        for name in names:
+            e = rel_err(getattr(g._layers[li], name), getattr(r._layers[li], name))
+            assert e <= tol, f"L{li}.{name}: {e:.3e} > {tol:.1e}"
+
+
+def _mask_diff(a, b):
+    return int((a != b).sum())
+
+
+def test_small_network_epochs_with_rewiring_f64(hb):
+    # 3 + 2 epochs, 13 batches with a short last one, rewiring from the second epoch on: in float64
+    # the whole trajectory, masks included, is reproduced.
+    (g, r), (Xt, Yt) = _run_both(hb, np.float64, n_pix=60, H=4, Mc=10, n_out=5, Ns=200, Nt=50, B=16,
+                                 e1=3, e2=2, hp=dict(MNIST_HP, l1_density=0.3), data_seed=11)
+    assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
+    _compare_states(g, r, 1e-10)
+    assert np.array_equal(g.predict(Xt, 16), r.predict(Xt, 16))
+    cg, tg = g.evaluate(Xt, Yt, 16)
+    cr, tr = r.evaluate(Xt, Yt, 16)
+    assert cg.tolist() == cr.tolist() and tg.tolist() == tr.tolist()
+
+
+def test_small_network_one_epoch_f32(hb):
+    # float32, one epoch per layer (13 batches, short last one).  Stated drift bound after one epoch:
+    # 1e-4 relative (rounding differences of ~1e-7 per step, amplified by the log of small traces).
+    (g, r), (Xt, Yt) = _run_both(hb, np.float32, n_pix=60, H=4, Mc=10, n_out=5, Ns=200, Nt=50, B=16,
+                                 e1=1, e2=1, hp=dict(MNIST_HP, l1_density=0.3), data_seed=11)
+    assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
+    _compare_states(g, r, 1e-4)
+    assert np.array_equal(g.predict(Xt, 16), r.predict(Xt, 16))
+
+
+def test_mnist_shape_one_epoch_f32(hb):
+    # MNIST shape (1568 -> 30x100 -> 10), float32, batch 128, 31 batches (short last one), one epoch
+    # per layer.  Stated drift bound after one epoch: 1e-4 relative; predicted labels bit-exact.
+    (g, r), (Xt, Yt) = _run_both(hb, np.float32, n_pix=784, H=30, Mc=100, n_out=10, Ns=31 * 128 - 32,
+                                 Nt=256, B=128, e1=1, e2=1, hp=MNIST_HP, data_seed=1001)
+    assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
+    _compare_states(g, r, 1e-4)
+    assert np.array_equal(g.predict(Xt, 128), r.predict(Xt, 128))
+    cg, _ = g.evaluate(Xt, Yt, 128)
+    cr, _ = r.evaluate(Xt, Yt, 128)
+    assert cg.tolist() == cr.tolist()
+
+
+def test_mnist_shape_rewiring_epoch_f32(hb):
+    # Second epoch, with rewiring (31 // 31 = 1: hypercolumns rewire on steps 0..29).  Over a float32
+    # TRAJECTORY mask equality is not well defined: each swap compares scores that are sums of
+    # nearly cancelling terms, so rounding-level state differences flip near-ties and the runs fork.
+    # The reference's own arithmetic shows it: the strict-IEEE and the -ffast-math build of the
+    # oracle disagree in 20 mask entries on this very run, and both disagree with float64.
+    # What holds, and is asserted: every decision is bit-exact given identical inputs
+    # (test_rewiring_decisions_replayed_f32), column popcounts are preserved, and most swaps agree.
+    (g, r), _ = _run_both(hb, np.float32, n_pix=784, H=30, Mc=100, n_out=10, Ns=31 * 128 - 32,
+                          Nt=8, B=128, e1=2, e2=0, hp=MNIST_HP, data_seed=1001)
+    gm, rm, init = g._layers[0].wmask, r._layers[0].wmask, build_init_mask()
+    changed = _mask_diff(rm, init)
+    assert changed > 500, "the run is meant to rewire"
+    assert np.array_equal(gm.sum(0), init.sum(0)) and np.array_equal(rm.sum(0), init.sum(0))
+    assert _mask_diff(gm, rm) <= 0.25 * changed, f"{_mask_diff(gm, rm)} of {changed} rewired entries differ"
+    assert np.all(np.isfinite(g._layers[0].weights))
+
+
+def test_rewiring_decisions_replayed_f32(hb):
+    # Every rewiring decision of a real float32 training run of the oracle (states after the trace and
+    # weight update of that step), replayed through the GPU kernel on identical inputs: bit-exact.
+    from oracle import cpu_backend as ob
+    from streambrain_amd import kernels_hip as k
+    captured = []
+
+    class Recorder(ob.StructuralPlasticityLayer):
+        def train_step(self, inputs, outputs, hypercolumn=None):
+            if hypercolumn is None:
+                return super().train_step(inputs, outputs, None)
+            cthr = self.taupdt / 2
+            self.k.update_weights(self.Ci, self.Cj, self.Cij, np.ascontiguousarray(inputs),
+                                  np.ascontiguousarray(outputs), self.taupdt, self.weights, cthr)
+            self.k.update_bias_regularized(self.bias, self.kbi, self.Cj, cthr, self.khalf, self.pmin,
+                                           self.taubdt)
+            before = self.wmask.copy()
+            self.k.update_mask(self.wmask, self.weights, self.Ci, self.Cj, self.Cij, cthr,
+                               self.hypercolumns, self.minicolumns, int(hypercolumn), 16)
+            captured.append((before, self.weights.copy(), self.Ci.copy(), self.Cj.copy(),
+                             self.Cij.copy(), cthr, int(hypercolumn), self.wmask.copy()))
+            self.k.apply_mask(self.weights, self.wmask, self.hypercolumns, self.minicolumns)
+
+    class Backend:
+        Network = ob.Network
+        StructuralPlasticityLayer = Recorder
+        DenseLayer = ob.DenseLayer
+
+    for n_pix, H, Mc, Ns, B, epochs, hp, seed in [
+            (60, 4, 10, 200, 16, 3, dict(MNIST_HP, l1_density=0.3), 11),
+            (784, 30, 100, 31 * 128 - 32, 128, 2, MNIST_HP, 1001)]:
+        captured.clear()
+        rng = np.random.default_rng(seed)
+        X, Y = synthetic_images(rng, Ns, n_pix), one_hot_labels(rng, Ns, 5)
+        net = build_two_layer(Backend, 2 * n_pix, H, Mc, 5, hp, np.float32, seed=0)
+        net.fit(X, Y, B, [(0, epochs)])
+        assert len(captured) >= min(H, 8)
+        swapped = 0
+        for before, W, Ci, Cj, Cij, cthr, h, after in captured:
+            got = k.update_mask(before.copy(), W, Ci, Cj, Cij, cthr, H, Mc, h, 16)
+            assert _mask_diff(got, after) == 0, f"hypercolumn {h}: {_mask_diff(got, after)} entries differ"
+            swapped += _mask_diff(before, after)
+        assert swapped > 0
+
+
+def build_init_mask():
+    np.random.seed(0)
+    np.random.randn(1568, 3000); np.random.rand(3000)
+    return (np.random.rand(1568, 30) < MNIST_HP["l1_density"]).astype(np.uint8)
+
+
+def test_zero_period_schedule_does_not_rewire(hb):
+    # 2 batches, 5 hypercolumns: 2 // 6 == 0.  The reference divides by zero here; this backend trains
+    # without rewiring.
+    rng = np.random.default_rng(3)
+    X, Y = synthetic_images(rng, 40, 30), one_hot_labels(rng, 40, 4)
+    net = build_two_layer(hb, 60, 5, 6, 4, MNIST_HP, np.float32, seed=0, density=0.3)
+    before = net._layers[0].wmask
+    net.fit(X, Y, 32, [(0, 3)])
+    assert np.array_equal(net._layers[0].wmask, before)
+    assert np.all(np.isfinite(net._layers[0].weights))
+
+
+def test_errors_are_python_exceptions(hb):
+    net = hb.Network(np.float32)
+    with pytest.raises(Exception):
+        hb.Network(np.int32)
+    net.add_layer(hb.DenseLayer(8, 1, 3, 0.01, (0.1, 0.3, 0.03)))
+    with pytest.raises(RuntimeError):
+        net.net.train_epoch(0, 4, np.arange(4), None, 0)  # no training data
+    with pytest.raises(RuntimeError):
+        net.net.get_layer_state(0, "kbi")  # dense layers have no kbi
+    with pytest.raises(RuntimeError):
+        net.net.set_layer_state(0, "weights", np.zeros((3, 3), np.float32))
