@@ -1,0 +1,234 @@
+#!/usr/bin/env python3
+"""Benchmark of the BCPNN layer training step on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+Workload (BASELINE.json configs[1]): MNIST-shaped 2-layer network, float32, batch 128, 60000 seeded
+synthetic samples; input 784 pixels complementary-coded to 1568 units (~19% nonzero pixels, uniform
+in (0,1]); hidden layer 30 hypercolumns x 100 minicolumns with a receptive-field mask of density 0.1;
+10-class dense output layer.  A "step" is one structural-plasticity-layer training step on one
+resident batch: forward x.W+b with per-hypercolumn softmax, Ci/Cj/Cij trace update, weight and bias
+recompute, mask apply, and the mask rewiring at the reference's cadence (every 15th step of an epoch
+after the first).  The timed region starts with the training set already in HBM.
+
+Prints one JSON line.  `value` is training samples/s; `roofline` describes the dominant kernel (the
+fused trace+weight pass); `cpu_baseline` is the CPU oracle (the reference's OpenMP loop structure,
+built with the reference's flag set) timed on this host on a bounded number of the same steps.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+N_PIXELS, H, MC, N_OUT, BATCH, N_SAMPLES = 784, 30, 100, 10, 128, 60000
+HP = dict(l1_taupdt=0.006908854922437549, l1_pmin=0.06195283356566607, l1_khalf=-139.02586632856327,
+          l1_taubdt=0.02218100432360414, l1_density=0.1, l2_taupdt=0.0007449780036161324)
+HBM_PEAK_GBS = 8000.0
+
+
+def synthetic_dataset(n, seed=1001):
+    rng = np.random.default_rng(seed)
+    px = (1.0 - rng.random((n, N_PIXELS), dtype=np.float32)) * (rng.random((n, N_PIXELS), dtype=np.float32) < 0.19)
+    x = np.concatenate([px, 1.0 - px], axis=1).astype(np.float32)
+    y = np.zeros((n, N_OUT), dtype=np.float32)
+    y[np.arange(n), rng.integers(0, N_OUT, n)] = 1.0
+    return x, y
+
+
+def initial_state(seed=0):
+    """Layer state drawn in the reference's order from numpy's legacy global stream."""
+    n, m = 2 * N_PIXELS, H * MC
+    np.random.seed(seed)
+    st = {
+        "weights": (0.1 * np.random.randn(n, m)).astype(np.float32),
+        "bias": (0.1 * np.random.rand(m)).astype(np.float32),
+        "Ci": np.ones(n, dtype=np.float32),
+        "Cj": np.full(m, 1.0 / MC, dtype=np.float32),
+        "Cij": np.full((n, m), 1.0 / MC, dtype=np.float32),
+        "kbi": np.ones(m, dtype=np.float32),
+    }
+    st["wmask"] = (np.random.rand(n, H) < HP["l1_density"]).astype(np.uint8)
+    return st
+
+
+def batch_plan(first_step, n_steps, nb):
+    """Splits a run of consecutive steps into per-epoch ranges (epoch, first_batch, n_batches);
+    epoch numbering starts at 1 so that the rewiring cadence is part of the measurement."""
+    out = []
+    step = first_step
+    left = n_steps
+    while left > 0:
+        epoch, fb = 1 + step // nb, step % nb
+        take = min(left, nb - fb)
+        out.append((epoch, fb, take))
+        step += take
+        left -= take
+    return out
+
+
+class GpuRun:
+    def __init__(self, x, y):
+        from streambrain_amd import _capi
+        self.capi = _capi
+        self.lib = _capi.lib()
+        _capi.init(0)
+        self.net = ctypes.c_void_p()
+        _capi.check(self.lib.sb_net_create(ctypes.byref(self.net), 0))
+        c = self.capi.check
+        c(self.lib.sb_net_add_plastic_layer(self.net, 2 * N_PIXELS, H, MC, HP["l1_taupdt"], HP["l1_pmin"],
+                                            HP["l1_khalf"], HP["l1_taubdt"], 1.0, 1.0 / MC, 1.0 / MC))
+        c(self.lib.sb_net_add_dense_layer(self.net, H * MC, 1, N_OUT, HP["l2_taupdt"], 1.0 / MC,
+                                          1.0 / N_OUT, 1.0 / MC / N_OUT))
+        for name, arr in initial_state().items():
+            arr = np.ascontiguousarray(arr)
+            c(self.lib.sb_net_set_layer_state(self.net, 0, name.encode(), arr.ctypes.data, arr.nbytes))
+        c(self.lib.sb_net_set_training_data(self.net, x.ctypes.data, y.ctypes.data, x.shape[0], x.shape[1],
+                                            y.shape[1]))
+        self.ns = x.shape[0]
+        self.nb = (self.ns + BATCH - 1) // BATCH
+        self.rng = np.random.default_rng(7)
+
+    def run_steps(self, first_step, n_steps):
+        """Enqueues steps [first_step, first_step + n_steps); returns the number of samples."""
+        samples = 0
+        for epoch, fb, take in batch_plan(first_step, n_steps, self.nb):
+            perm = self.rng.permutation(self.ns).astype(np.int64) if fb == 0 else None
+            hc = self.rng.permutation(H).astype(np.int64)
+            if fb != 0 and not getattr(self, "_laid_out", False):
+                # a run that starts mid-epoch still needs the epoch's sample order applied once
+                perm0 = self.rng.permutation(self.ns).astype(np.int64)
+                self.capi.check(self.lib.sb_net_train_batches(self.net, 0, BATCH, perm0.ctypes.data,
+                                                              hc.ctypes.data, epoch, 0, 0, 0))
+            self._laid_out = True
+            self.capi.check(self.lib.sb_net_train_batches(
+                self.net, 0, BATCH, perm.ctypes.data if perm is not None else None, hc.ctypes.data,
+                epoch, fb, take, 0))
+            for b in range(fb, fb + take):
+                samples += min(BATCH, self.ns - b * BATCH)
+        return samples
+
+    def sync(self):
+        self.capi.check(self.lib.sb_sync())
+
+    def profile(self, first_step, n_steps):
+        self.capi.check(self.lib.sb_profile_start())
+        self.run_steps(first_step, n_steps)
+        self.capi.check(self.lib.sb_profile_stop())
+        out = {}
+        for k in range(self.lib.sb_profile_kernels()):
+            ms, n = ctypes.c_double(0), ctypes.c_long(0)
+            self.capi.check(self.lib.sb_profile_get(k, ctypes.byref(ms), ctypes.byref(n)))
+            if n.value:
+                out[self.lib.sb_profile_kernel_name(k).decode()] = {
+                    "launches": n.value, "avg_us": 1e3 * ms.value / n.value}
+        return out
+
+
+def cpu_baseline(x, y, budget_s=20.0, max_steps=40):
+    """The CPU oracle (reference loop structure, reference flag set, OpenMP) on the first steps of the
+    same workload: same initial state, same data, batches in storage order, rewiring every 15th step."""
+    from oracle.oracle import Oracle
+    o = Oracle(fast=True)
+    st = initial_state()
+    tau, cthr = HP["l1_taupdt"], HP["l1_taupdt"] / 2
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+
+    def step(i):
+        xb = x[i * BATCH:(i + 1) * BATCH]
+        act = np.zeros((xb.shape[0], H * MC), dtype=np.float32)
+        o.update_state(act, st["weights"], st["bias"], xb)
+        o.softmax_minicolumns(act, H, MC)
+        o.update_weights(st["Ci"], st["Cj"], st["Cij"], xb, act, tau, st["weights"], cthr)
+        o.update_bias_regularized(st["bias"], st["kbi"], st["Cj"], cthr, HP["l1_khalf"], HP["l1_pmin"],
+                                  HP["l1_taubdt"])
+        if i % 15 == 0 and i // 15 < H:
+            o.update_mask(st["wmask"], st["weights"], st["Ci"], st["Cj"], st["Cij"], cthr, H, MC, i // 15, 16)
+        o.apply_mask(st["weights"], st["wmask"], H, MC)
+        return xb.shape[0]
+
+    step(0)  # warm-up (thread pool, page faults)
+    t0 = time.perf_counter()
+    samples = steps = 0
+    while steps < max_steps and time.perf_counter() - t0 < budget_s:
+        samples += step(1 + steps)
+        steps += 1
+    dt = time.perf_counter() - t0
+    return {"value": samples / dt, "unit": "samples/s", "cores": threads, "kind": "port",
+            "sample": f"{steps} training steps of the same workload (batch {BATCH}, rewiring every 15th step), "
+                      f"{dt:.1f} s, oracle built -O3 -march=x86-64-v3 -ffast-math -fopenmp",
+            "ms_per_step": 1e3 * dt / max(steps, 1)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=938)
+    ap.add_argument("--warmup", type=int, default=60)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--samples", type=int, default=N_SAMPLES)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
+              "(the path is not sharded across devices)", file=sys.stderr)
+        return 2
+
+    x, y = synthetic_dataset(args.samples)
+    run = GpuRun(x, y)
+
+    run.run_steps(0, args.warmup)
+    run.sync()
+    t0 = time.perf_counter()
+    samples = run.run_steps(args.warmup, args.steps)
+    run.sync()
+    dt = time.perf_counter() - t0
+
+    prof = run.profile(args.warmup + args.steps, min(args.steps, 2 * run.nb))
+    n, m = 2 * N_PIXELS, H * MC
+    tw = prof.get("trace_weights", {"avg_us": float("nan")})
+    alg_bytes = 3 * 4 * n * m  # read Cij, write Cij, write W: 12 bytes per synapse
+    achieved = alg_bytes / (tw["avg_us"] * 1e-6) / 1e9
+    fwd = prof.get("forward", {"avg_us": float("nan")})
+    fwd_tflops = 2.0 * BATCH * n * m / (fwd["avg_us"] * 1e-6) / 1e12
+
+    result = {
+        "metric": "train samples/sec on 1 MI355X (MNIST-shape fp32 b128); % HBM / MFMA peak",
+        "value": samples / dt,
+        "unit": "samples/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": 1e3 * dt / args.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: MNIST-shaped 2-layer network, structural-plasticity layer "
+                               "training steps (1568 -> 30x100, mask density 0.1, rewiring every 15th step)",
+                   "batch": BATCH, "in_features": n, "hypercolumns": H, "minicolumns": MC,
+                   "samples": args.samples},
+        "roofline": {"bound": "hbm", "kernel": "k_trace_weights", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": tw["avg_us"]},
+        "mfma": {"kernel": "k_forward", "achieved_tflops": fwd_tflops, "peak_tflops": 157.3,
+                 "frac": fwd_tflops / 157.3, "avg_launch_us": fwd["avg_us"],
+                 "trace_gemm_tflops_in_fused_kernel": 2.0 * BATCH * n * m / (tw["avg_us"] * 1e-6) / 1e12},
+        "kernels": prof,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(x, y)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

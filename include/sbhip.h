@@ -179,6 +179,14 @@ int sb_net_training_done(sb_net *net);
 int sb_net_train_epoch(sb_net *net, int layer, long maximal_batch_size,
                        const int64_t *h_sample_perm, const int64_t *h_hc_perm, long epoch_index);
 
+/* A contiguous range of an epoch's batches [first_batch, first_batch + n_batches): sb_net_train_epoch
+ * is the whole range with finalize = 1.  The sample order is applied when first_batch == 0 (it may be
+ * NULL otherwise); later ranges continue the same epoch.  For callers that interleave their own work
+ * (progress reporting as in _cpu_base_backend.py:270-312, timing) with an epoch. */
+int sb_net_train_batches(sb_net *net, int layer, long maximal_batch_size,
+                         const int64_t *h_sample_perm, const int64_t *h_hc_perm, long epoch_index,
+                         long first_batch, long n_batches, int finalize);
+
 /* Network.evaluate (_cpu_base_backend.py:205-245): forward through every layer, count rows whose
  * argmax equals the label's argmax.  Synchronous.  h_pred (may be NULL) receives the predicted
  * class per row. */
@@ -195,6 +203,17 @@ int sb_net_predict(sb_net *net, const void *h_images, long n_samples, long n_fea
  * last_layer [n_rows, M_last] is copied to h_act.  Synchronous. */
 int sb_net_forward(sb_net *net, const void *h_images, long n_rows, long n_features, int last_layer,
                    long maximal_batch_size, void *h_act);
+
+/* ---- per-kernel timing -------------------------------------------------------------------------
+ * Between sb_profile_start and sb_profile_stop every kernel launch of the library is bracketed by HIP
+ * events on the library's stream; afterwards sb_profile_get returns, per kernel index in
+ * [0, sb_profile_kernels()), the summed elapsed time and the number of launches.  The reference has no
+ * counterpart (it times whole runs with time.time(), train.py:181-193). */
+int sb_profile_start(void);
+int sb_profile_stop(void);
+int sb_profile_kernels(void);
+const char *sb_profile_kernel_name(int kernel);
+int sb_profile_get(int kernel, double *total_ms, long *launches);
 
 #ifdef __cplusplus
 }

@@ -51,17 +51,23 @@ _PLAIN_SIGS = {
     "sb_net_set_training_data": [_P, _P, _P, _L, _L, _L],
     "sb_net_training_done": [_P],
     "sb_net_train_epoch": [_P, _I, _L, _P, _P, _L],
+    "sb_net_train_batches": [_P, _I, _L, _P, _P, _L, _L, _L, _I],
+    "sb_profile_start": [],
+    "sb_profile_stop": [],
+    "sb_profile_kernels": [],
+    "sb_profile_get": [_I, ctypes.POINTER(_D), ctypes.POINTER(_L)],
     "sb_net_evaluate": [_P, _P, _P, _L, _L, _L, _L, ctypes.POINTER(ctypes.c_int64),
                         ctypes.POINTER(ctypes.c_int64), _P],
     "sb_net_predict": [_P, _P, _L, _L, _L, _P],
     "sb_net_forward": [_P, _P, _L, _L, _I, _L, _P],
 }
 _RESTYPES = {"sb_last_error": ctypes.c_char_p, "sb_stream": _P}
+_OTHER_SIGS = {"sb_profile_kernel_name": ([_I], ctypes.c_char_p)}
 
 
 def exported_symbols():
     """Every symbol include/sbhip.h declares."""
-    names = list(_PLAIN_SIGS) + list(_RESTYPES)
+    names = list(_PLAIN_SIGS) + list(_RESTYPES) + list(_OTHER_SIGS)
     for base in _KERNEL_SIGS:
         names += [base + "_f32", base + "_f64"]
     return names
@@ -85,6 +91,10 @@ def lib():
         for name, res in _RESTYPES.items():
             f = getattr(L, name)
             f.argtypes = []
+            f.restype = res
+        for name, (args, res) in _OTHER_SIGS.items():
+            f = getattr(L, name)
+            f.argtypes = args
             f.restype = res
         for base, sig in _KERNEL_SIGS.items():
             for sfx, R in (("_f32", _F), ("_f64", _D)):

@@ -27,6 +27,20 @@ struct TraceScalars {
   }
 };
 
+// Per-kernel timing: when profiling is on (sb_profile_start), every launcher brackets its launches
+// with a pair of HIP events on the launch stream; sb_profile_stop sums the elapsed times per kernel.
+enum KernelId {
+  K_FORWARD = 0, K_SOFTMAX, K_COUNTERS, K_TRACE_WEIGHTS, K_UPDATE_BIAS, K_UPDATE_BIAS_REG, K_MASK_SCORES,
+  K_MASK_SWAP, K_MASK_FIX, K_APPLY_MASK, K_ARGMAX, K_GATHER, K_FILL, K_COUNT
+};
+const char *kernel_name(int id);
+struct ProfScope {
+  ProfScope(hipStream_t st, int id);
+  ~ProfScope();
+  hipStream_t st_;
+  int slot_;
+};
+
 void set_error(const std::string &msg);
 int hip_fail(hipError_t e, const char *what, const char *file, int line);
 

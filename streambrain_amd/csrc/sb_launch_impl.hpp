@@ -14,6 +14,7 @@ static inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 // ------------------------------------------------------------------------------------------- forward
 template <typename T, int NG, bool FUSE>
 static int forward_variant(hipStream_t st, const ForwardArgs<T> &a, dim3 grid, bool vec) {
+  ProfScope prof_(st, K_FORWARD);
   if (vec)
     hipLaunchKernelGGL((k_forward<T, NG, FUSE, true>), grid, dim3(256), 0, st, a);
   else
@@ -59,6 +60,7 @@ int launch_softmax(hipStream_t st, T *act, long B, long H, long Mc) {
   SB_REQUIRE(B > 0 && H > 0 && Mc > 0, "sizes must be positive");
   const long groups = B * H;
   SB_REQUIRE(cdiv(groups, 4) < (1L << 31), "too many groups");
+  ProfScope prof_(st, K_SOFTMAX);
   hipLaunchKernelGGL((k_softmax<T>), dim3((unsigned)cdiv(groups, 4)), dim3(256), 0, st, act, groups,
                      Mc);
   SB_LAUNCH_CHECK();
@@ -77,6 +79,7 @@ int launch_counters(hipStream_t st, const T *x, const T *y, T *Ci, T *Cj, long B
   a.tau = taupdt; a.omt = (T)(1.0 - (double)taupdt); a.fB = (T)B;
   a.bias_mode = bias_mode; a.bias = bias; a.kbi = kbi;
   a.cthr = cthr; a.khalf = khalf; a.pmin = pmin; a.taubdt = taubdt;
+  ProfScope prof_(st, K_COUNTERS);
   hipLaunchKernelGGL((k_counters<T>), dim3((unsigned)cdiv(N + M, 256)), dim3(256), 0, st, a);
   SB_LAUNCH_CHECK();
   return 0;
@@ -91,6 +94,7 @@ static int trace_variant(hipStream_t st, const TraceArgs<T> &a, bool vec) {
     set_error("launch_trace_weights: in_features too large for one launch");
     return -1;
   }
+  ProfScope prof_(st, K_TRACE_WEIGHTS);
   if (vec)
     hipLaunchKernelGGL((k_trace_weights<T, RX, RY, true, true>), grid, dim3(256), 0, st, a);
   else
@@ -126,6 +130,7 @@ template <typename T>
 int launch_update_bias(hipStream_t st, T *bias, const T *Cj, T cthr, long M) {
   SB_REQUIRE(bias && Cj, "null pointer");
   SB_REQUIRE(M > 0, "sizes must be positive");
+  ProfScope prof_(st, K_UPDATE_BIAS);
   hipLaunchKernelGGL((k_update_bias<T>), dim3((unsigned)cdiv(M, 256)), dim3(256), 0, st, bias, Cj, cthr,
                      M);
   SB_LAUNCH_CHECK();
@@ -137,6 +142,7 @@ int launch_update_bias_regularized(hipStream_t st, T *bias, T *kbi, const T *Cj,
                                    T pmin, T taubdt, long M) {
   SB_REQUIRE(bias && kbi && Cj, "null pointer");
   SB_REQUIRE(M > 0, "sizes must be positive");
+  ProfScope prof_(st, K_UPDATE_BIAS_REG);
   hipLaunchKernelGGL((k_update_bias_regularized<T>), dim3((unsigned)cdiv(M, 256)), dim3(256), 0, st,
                      bias, kbi, Cj, cthr, khalf, pmin, taubdt, M);
   SB_LAUNCH_CHECK();
@@ -158,9 +164,13 @@ int launch_update_mask(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, 
   a.wmask = wmask; a.W = W; a.Ci = Ci; a.Cj = Cj; a.Cij = Cij; a.cthr = cthr; a.cthr4 = s.cthr4;
   a.N = N; a.M = H * Mc; a.H = H; a.Mc = Mc; a.h = h; a.iterations = iterations; a.nom = nom;
   a.csum = csum;
-  hipLaunchKernelGGL((k_mask_scores<T>), dim3((unsigned)cdiv(N, 4)), dim3(256), 0, st, a);
-  SB_LAUNCH_CHECK();
+  {
+    ProfScope prof_(st, K_MASK_SCORES);
+    hipLaunchKernelGGL((k_mask_scores<T>), dim3((unsigned)cdiv(N, 4)), dim3(256), 0, st, a);
+    SB_LAUNCH_CHECK();
+  }
   if (iterations > 0) {
+    ProfScope prof_(st, K_MASK_SWAP);
     hipLaunchKernelGGL((k_mask_swap<T>), dim3(1), dim3(1024), 0, st, a);
     SB_LAUNCH_CHECK();
   }
@@ -173,6 +183,7 @@ int launch_mask_fix_weights(hipStream_t st, T *W, const uint8_t *wmask, const T 
   SB_REQUIRE(W && wmask && Ci && Cj && Cij, "null pointer");
   SB_REQUIRE(h >= 0 && h < H, "hypercolumn index out of range");
   const TraceScalars<T> s = TraceScalars<T>::from(T(0), cthr);
+  ProfScope prof_(st, K_MASK_FIX);
   hipLaunchKernelGGL((k_mask_fix_weights<T>), dim3((unsigned)cdiv(N * Mc, 256)), dim3(256), 0, st, W,
                      wmask, Ci, Cj, Cij, cthr, s.cthr4, N, H * Mc, H, Mc, h);
   SB_LAUNCH_CHECK();
@@ -185,6 +196,7 @@ int launch_apply_mask(hipStream_t st, T *W, const uint8_t *wmask, long N, long H
   SB_REQUIRE(N > 0 && H > 0 && Mc > 0, "sizes must be positive");
   const long total = N * H * Mc;
   const long blocks = cdiv(total, 256) < 8192 ? cdiv(total, 256) : 8192;
+  ProfScope prof_(st, K_APPLY_MASK);
   hipLaunchKernelGGL((k_apply_mask<T>), dim3((unsigned)blocks), dim3(256), 0, st, W, wmask, N, H * Mc,
                      H, Mc);
   SB_LAUNCH_CHECK();
@@ -198,6 +210,7 @@ int launch_argmax_rows(hipStream_t st, const T *act, const T *labels, long B, lo
   SB_REQUIRE(act, "null pointer");
   SB_REQUIRE(!labels || correct, "labels need a counter");
   SB_REQUIRE(B > 0 && M > 0, "sizes must be positive");
+  ProfScope prof_(st, K_ARGMAX);
   hipLaunchKernelGGL((k_argmax_rows<T>), dim3((unsigned)cdiv(B, 4)), dim3(256), 0, st, act, labels, B,
                      M, pred, correct);
   SB_LAUNCH_CHECK();
@@ -209,6 +222,7 @@ int launch_gather_rows(hipStream_t st, T *dst, const T *src, const int64_t *idx,
                        long cols) {
   SB_REQUIRE(dst && src && idx, "null pointer");
   SB_REQUIRE(rows > 0 && cols > 0 && rows < (1L << 31), "bad shape");
+  ProfScope prof_(st, K_GATHER);
   hipLaunchKernelGGL((k_gather_rows<T>), dim3((unsigned)rows), dim3(256), 0, st, dst, src, idx, rows,
                      cols);
   SB_LAUNCH_CHECK();
@@ -220,6 +234,7 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
   if (n == 0) return 0;
   SB_REQUIRE(dst, "null pointer");
   const size_t blocks = (n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096;
+  ProfScope prof_(st, K_FILL);
   hipLaunchKernelGGL((k_fill<T>), dim3((unsigned)blocks), dim3(256), 0, st, dst, value, n);
   SB_LAUNCH_CHECK();
   return 0;

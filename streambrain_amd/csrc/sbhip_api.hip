@@ -32,6 +32,47 @@ struct Context {
 static Context g_ctx;
 static std::mutex g_ctx_mutex;
 
+// ---- per-kernel event timing (sb_profile_start / sb_profile_stop)
+struct ProfRecord {
+  int id;
+  hipEvent_t start, stop;
+};
+static bool g_prof_on = false;
+static std::vector<ProfRecord> g_prof_records;
+static std::vector<hipEvent_t> g_prof_pool;
+static double g_prof_ms[K_COUNT];
+static long g_prof_launches[K_COUNT];
+
+const char *kernel_name(int id) {
+  static const char *names[K_COUNT] = {"forward", "softmax", "counters", "trace_weights", "update_bias",
+                                       "update_bias_regularized", "mask_scores", "mask_swap",
+                                       "mask_fix_weights", "apply_mask", "argmax", "gather_rows", "fill"};
+  return (id >= 0 && id < K_COUNT) ? names[id] : "?";
+}
+
+static hipEvent_t prof_event() {
+  hipEvent_t e = nullptr;
+  if (!g_prof_pool.empty()) {
+    e = g_prof_pool.back();
+    g_prof_pool.pop_back();
+  } else if (hipEventCreate(&e) != hipSuccess) {
+    e = nullptr;
+  }
+  return e;
+}
+
+ProfScope::ProfScope(hipStream_t st, int id) : st_(st), slot_(-1) {
+  if (!g_prof_on) return;
+  ProfRecord r{id, prof_event(), prof_event()};
+  if (!r.start || !r.stop) return;
+  (void)hipEventRecord(r.start, st);
+  g_prof_records.push_back(r);
+  slot_ = (int)g_prof_records.size() - 1;
+}
+ProfScope::~ProfScope() {
+  if (slot_ >= 0) (void)hipEventRecord(g_prof_records[slot_].stop, st_);
+}
+
 static int require_ready() {
   if (!g_ctx.ready) {
     set_error("sb_init has not been called");
@@ -176,8 +217,9 @@ static int layer_train_step(Layer &L, const T *x, const T *y, long B, long h) {
 }
 
 template <typename T>
-static int net_train_epoch(sb_net *net, int layer, long maxB, const int64_t *h_sample_perm,
-                           const int64_t *h_hc_perm, long epoch) {
+static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h_sample_perm,
+                             const int64_t *h_hc_perm, long epoch, long first_batch, long n_batches,
+                             bool finalize) {
   hipStream_t st = g_ctx.stream;
   Layer &target = net->layers[layer];
   const bool last = layer + 1 == (int)net->layers.size();
@@ -188,10 +230,16 @@ static int net_train_epoch(sb_net *net, int layer, long maxB, const int64_t *h_s
   for (int l = 1; l <= layer; l++)
     SB_REQUIRE(net->layers[l].N == net->layers[l - 1].M, "layer widths do not chain");
   const long Ns = net->Ns;
-  for (long r = 0; r < Ns; r++)
-    SB_REQUIRE(h_sample_perm[r] >= 0 && h_sample_perm[r] < Ns, "sample index out of range");
+  const long nb = (Ns + maxB - 1) / maxB;
+  SB_REQUIRE(first_batch >= 0 && n_batches >= 0 && first_batch + n_batches <= nb, "batch range");
   int rc = ensure_act(net, maxB < Ns ? maxB : Ns);
   if (rc) return rc;
+  const bool permute = first_batch == 0;  // a later range continues the epoch already laid out
+  SB_REQUIRE(permute || net->Xp, "the epoch's first batches have not been run");
+  if (permute) {
+  SB_REQUIRE(h_sample_perm, "sample order missing");
+  for (long r = 0; r < Ns; r++)
+    SB_REQUIRE(h_sample_perm[r] >= 0 && h_sample_perm[r] < Ns, "sample index out of range");
 
   // images[idx, :] / labels[idx, :]  (_cpu_base_backend.py:258-260)
   if (!net->Xp) SB_HIP(hipMalloc(&net->Xp, (size_t)Ns * net->NF * net->esize));
@@ -206,10 +254,10 @@ static int net_train_epoch(sb_net *net, int layer, long maxB, const int64_t *h_s
   if (last)
     if ((rc = launch_gather_rows<T>(st, (T *)net->Yp, (const T *)net->Y, net->d_perm, Ns, net->NC)))
       return rc;
+  }
 
-  const long nb = (Ns + maxB - 1) / maxB;
   const long period = nb / (target.H + 1);  // _cpu_base_backend.py:297-299
-  for (long i = 0; i < nb; i++) {
+  for (long i = first_batch; i < first_batch + n_batches; i++) {
     const long lo = i * maxB;
     const long B = (lo + maxB <= Ns) ? maxB : Ns - lo;
     const T *x = (const T *)net->Xp + lo * net->NF;
@@ -237,7 +285,7 @@ static int net_train_epoch(sb_net *net, int layer, long maxB, const int64_t *h_s
     if (rc) return rc;
   }
   // train_finalize, once per epoch (_cpu_base_backend.py:314; cpu_backend.py:17-18)
-  if (!target.plastic)
+  if (finalize && !target.plastic)
     return launch_update_bias<T>(st, (T *)target.bias, (const T *)target.Cj, (T)(target.taupdt / 2),
                                  target.M);
   return 0;
@@ -627,21 +675,76 @@ int sb_net_set_training_data(sb_net *net, const void *h_images, const void *h_la
   return 0;
 }
 
-int sb_net_train_epoch(sb_net *net, int layer, long maximal_batch_size, const int64_t *h_sample_perm,
-                       const int64_t *h_hc_perm, long epoch_index) {
+int sb_net_train_batches(sb_net *net, int layer, long maximal_batch_size,
+                         const int64_t *h_sample_perm, const int64_t *h_hc_perm, long epoch_index,
+                         long first_batch, long n_batches, int finalize) {
   SB_READY();
-  SB_REQUIRE(net && h_sample_perm, "null pointer");
+  SB_REQUIRE(net, "null pointer");
   if (!net->X) {
-    set_error("sb_net_train_epoch: no training data (call sb_net_set_training_data)");
+    set_error("sb_net_train_batches: no training data (call sb_net_set_training_data)");
     return SB_ERR_STATE;
   }
   SB_REQUIRE(layer >= 0 && layer < (int)net->layers.size(), "layer index out of range");
   SB_REQUIRE(maximal_batch_size > 0, "batch size must be positive");
   SB_REQUIRE(epoch_index >= 0, "epoch index must be non-negative");
   return net->dtype == SB_F32
-             ? net_train_epoch<float>(net, layer, maximal_batch_size, h_sample_perm, h_hc_perm, epoch_index)
-             : net_train_epoch<double>(net, layer, maximal_batch_size, h_sample_perm, h_hc_perm,
-                                       epoch_index);
+             ? net_train_batches<float>(net, layer, maximal_batch_size, h_sample_perm, h_hc_perm,
+                                        epoch_index, first_batch, n_batches, finalize != 0)
+             : net_train_batches<double>(net, layer, maximal_batch_size, h_sample_perm, h_hc_perm,
+                                         epoch_index, first_batch, n_batches, finalize != 0);
+}
+
+int sb_net_train_epoch(sb_net *net, int layer, long maximal_batch_size, const int64_t *h_sample_perm,
+                       const int64_t *h_hc_perm, long epoch_index) {
+  SB_READY();
+  SB_REQUIRE(net && h_sample_perm, "null pointer");
+  SB_REQUIRE(maximal_batch_size > 0, "batch size must be positive");
+  const long nb = net->Ns > 0 ? (net->Ns + maximal_batch_size - 1) / maximal_batch_size : 0;
+  return sb_net_train_batches(net, layer, maximal_batch_size, h_sample_perm, h_hc_perm, epoch_index, 0,
+                              nb, 1);
+}
+
+int sb_profile_start(void) {
+  SB_READY();
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  for (auto &r : g_prof_records) {
+    g_prof_pool.push_back(r.start);
+    g_prof_pool.push_back(r.stop);
+  }
+  g_prof_records.clear();
+  for (int k = 0; k < K_COUNT; k++) {
+    g_prof_ms[k] = 0;
+    g_prof_launches[k] = 0;
+  }
+  g_prof_on = true;
+  return 0;
+}
+
+int sb_profile_stop(void) {
+  SB_READY();
+  g_prof_on = false;
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  for (auto &r : g_prof_records) {
+    float ms = 0;
+    SB_HIP(hipEventElapsedTime(&ms, r.start, r.stop));
+    g_prof_ms[r.id] += ms;
+    g_prof_launches[r.id] += 1;
+    g_prof_pool.push_back(r.start);
+    g_prof_pool.push_back(r.stop);
+  }
+  g_prof_records.clear();
+  return 0;
+}
+
+int sb_profile_kernels(void) { return K_COUNT; }
+
+const char *sb_profile_kernel_name(int kernel) { return kernel_name(kernel); }
+
+int sb_profile_get(int kernel, double *total_ms, long *launches) {
+  SB_REQUIRE(kernel >= 0 && kernel < K_COUNT && total_ms && launches, "bad argument");
+  *total_ms = g_prof_ms[kernel];
+  *launches = g_prof_launches[kernel];
+  return 0;
 }
 
 int sb_net_evaluate(sb_net *net, const void *h_images, const void *h_labels, long n_samples,
