@@ -191,7 +191,7 @@ def main():
 
     prof = run.profile(args.warmup + args.steps, min(args.steps, 2 * run.nb))
     n, m = 2 * N_PIXELS, H * MC
-    tw = prof.get("trace_weights", {"avg_us": float("nan")})
+    tw = prof.get("train_fused") or prof.get("trace_weights") or {"avg_us": float("nan")}
     alg_bytes = 3 * 4 * n * m  # read Cij, write Cij, write W: 12 bytes per synapse
     achieved = alg_bytes / (tw["avg_us"] * 1e-6) / 1e9
     fwd = prof.get("forward", {"avg_us": float("nan")})
@@ -214,7 +214,7 @@ def main():
                                "training steps (1568 -> 30x100, mask density 0.1, rewiring every 15th step)",
                    "batch": BATCH, "in_features": n, "hypercolumns": H, "minicolumns": MC,
                    "samples": args.samples},
-        "roofline": {"bound": "hbm", "kernel": "k_trace_weights", "achieved": achieved, "peak": HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "k_train_fused", "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": tw["avg_us"]},
         "mfma": {"kernel": "k_forward", "achieved_tflops": fwd_tflops, "peak_tflops": 157.3,

@@ -29,6 +29,11 @@ struct Real<float> {
   }
   static __device__ __forceinline__ int acc_row(int q, int v) { return 4 * q + v; }
   static __device__ __forceinline__ float log_(float x) { return logf(x); }
+  // log for the weight recompute: the hardware log2 (1 ulp, v_log_f32) scaled by ln 2; arguments
+  // below the normal range, where that instruction flushes, take the library routine
+  static __device__ __forceinline__ float wlog(float x) {
+    return x >= 1.17549435e-38f ? __builtin_amdgcn_logf(x) * 0.693147180559945309f : logf(x);
+  }
   static __device__ __forceinline__ float exp_(float x) { return expf(x); }
   // single IEEE operations: the pragma keeps the compiler from contracting them into FMAs
   static __device__ __forceinline__ float add(float a, float b) {
@@ -55,6 +60,7 @@ struct Real<double> {
   }
   static __device__ __forceinline__ int acc_row(int q, int v) { return 4 * v + q; }
   static __device__ __forceinline__ double log_(double x) { return log(x); }
+  static __device__ __forceinline__ double wlog(double x) { return log(x); }
   static __device__ __forceinline__ double exp_(double x) { return exp(x); }
   static __device__ __forceinline__ double add(double a, double b) {
 #pragma clang fp contract(off)
@@ -105,6 +111,52 @@ __device__ __forceinline__ void store_vw(const T (&in)[Real<T>::VW], T *row, lon
   }
 }
 
+// Branch-free load for software-pipelined loops: the 16-byte load is always issued (from `p` when ok,
+// from the always-valid, 16-byte aligned `safe` otherwise) and the result zeroed afterwards, so the
+// compiler keeps several of them in flight with exact wait counts instead of fencing a guarded load.
+template <typename T>
+__device__ __forceinline__ void load_vw_sel(T (&out)[Real<T>::VW], const T *p, const T *safe, bool ok) {
+  constexpr int VW = Real<T>::VW;
+  const typename Real<T>::vec_t v = *reinterpret_cast<const typename Real<T>::vec_t *>(ok ? p : safe);
+#pragma unroll
+  for (int e = 0; e < VW; e++) out[e] = ok ? v[e] : T(0);
+}
+
+// Width-generic variants: W consecutive elements (W = 1, 2, 4 for float; 1, 2 for double), moved as one
+// W*sizeof(T)-byte access when VEC promises that alignment and limit % W == 0.
+template <typename T, int W>
+struct VecOf {
+  typedef T type __attribute__((ext_vector_type(W)));
+};
+template <typename T, int W, bool VEC>
+__device__ __forceinline__ void load_w(T (&out)[W], const T *row, long col, long limit, bool row_ok) {
+  if (VEC && W > 1) {
+    typename VecOf<T, (W > 1 ? W : 2)>::type v = {};
+    if (row_ok && col < limit)
+      v = *reinterpret_cast<const typename VecOf<T, (W > 1 ? W : 2)>::type *>(row + col);
+#pragma unroll
+    for (int e = 0; e < W; e++) out[e] = v[e];
+  } else {
+#pragma unroll
+    for (int e = 0; e < W; e++) out[e] = (row_ok && col + e < limit) ? row[col + e] : T(0);
+  }
+}
+template <typename T, int W, bool VEC>
+__device__ __forceinline__ void store_w(const T (&in)[W], T *row, long col, long limit) {
+  if (VEC && W > 1) {
+    if (col < limit) {
+      typename VecOf<T, (W > 1 ? W : 2)>::type v;
+#pragma unroll
+      for (int e = 0; e < W; e++) v[e] = in[e];
+      *reinterpret_cast<typename VecOf<T, (W > 1 ? W : 2)>::type *>(row + col) = v;
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < W; e++)
+      if (col + e < limit) row[col + e] = in[e];
+  }
+}
+
 // The weight of one synapse from its traces, shared by the trace/weight kernel and the rewiring
 // kernels so both see bit-identical values:  log(max(cij, cthr^4) / (ci * cj)) evaluated as
 // log(max(cij, cthr^4) * (1/ci) * (1/cj)).  rci / rcj are the reciprocals, or a negative number when
@@ -116,7 +168,7 @@ __device__ __forceinline__ T trace_reciprocal(T c, T cthr) {
 template <typename T>
 __device__ __forceinline__ T weight_from_traces(T cij, T rci, T rcj, T cthr4) {
   const T num = cij > cthr4 ? cij : cthr4;
-  const T w = Real<T>::log_(num * rci * rcj);
+  const T w = Real<T>::wlog(num * rci * rcj);
   return (rci < T(0) || rcj < T(0)) ? T(0) : w;
 }
 

@@ -1,0 +1,245 @@
+// Fused training pass of one layer: Ci / Cj / Cij moving averages, weight recompute, regularised bias
+// and mask apply in ONE kernel.                          omp.cc:89-205 (+ :222-246, :322-335)
+// ("omp.cc" = BCPNN/backend/_kernels/kernels_openmp_internal.cc of the reference)
+//
+//   Ci  <- max(0, Ci*(1-t) + mean_b x[b,i] * t)           Cj likewise from y
+//   Cij <- max(0, Cij*(1-t) + (x^T y / B) * t)
+//   W   <- wmask ? log(max(Cij, cthr^4) / (Ci*Cj)) : 0     (0 as well where Ci < cthr or Cj < cthr)
+//   bias/kbi <- update_bias_regularized(Cj)                (plastic layers)
+// all from the NEW traces, as the reference's fused loop does.
+//
+// A workgroup (256 threads, 4 wavefronts) owns a 64 x 64 tile of Cij.
+//   1. It requests its Cij tile right away (16-byte vectors, 256 contiguous bytes per 16 threads), so
+//      the HBM latency of the stream hides behind everything that follows.
+//   2. Per chunk of KCH batch rows it stages x[:, i-tile] and y[:, j-tile] in LDS with all loads in
+//      flight at once.  x and y are "k-major" in memory, which is the 16x16x4 MFMA operand layout, so
+//      staging is a plain copy and each wavefront feeds its 32 x 32 sub-tile (2 x 2 MFMA blocks) with
+//      two 8-byte LDS reads per K step of 4.
+//   3. From the same LDS slabs, 32 lanes of each wavefront add up one column each of x (resp. y) in
+//      batch order b = 0..B-1 without FMA contraction: the reference's summation order, so Ci, Cj and
+//      kbi stay bit-exact against a strict-IEEE build of it.  Every tile needs Ci for its rows and Cj
+//      for its columns, so every workgroup recomputes them from the OLD traces (a tile row shares x,
+//      a tile column shares y: same inputs, same order, same bits).  The old traces are read from
+//      Ci/Cj and the new ones written to Ci_next/Cj_next by the tiles of the first tile column / row:
+//      no workgroup ever reads a value another one is writing.
+//   4. The accumulators go through LDS into a row-major layout; each thread then finishes 4 consecutive
+//      columns of 4 rows: decay + clamp, weight, mask, one 16-byte store each to Cij and W.
+#pragma once
+#include "sb_kernels.hpp"
+
+namespace sb {
+
+template <typename T>
+struct TrainArgs {
+  const T *x;  // [B,N]
+  const T *y;  // [B,M]
+  T *Cij;
+  T *W;
+  const T *Ci;   // old traces (read)
+  const T *Cj;
+  T *Ci_next;    // new traces (written by the first tile column / row)
+  T *Cj_next;
+  const uint8_t *wmask;  // [N,H] or nullptr (no mask: every synapse active)
+  int bias_mode;         // 0: leave bias alone; 1: update_bias_regularized on the new Cj
+  T *bias, *kbi;
+  long B, N, M, H, Mc;
+  T tau, omt, fB, invB, cthr, cthr4;
+  T khalf, pmin, taubdt;
+  long tiles_i, tiles_j;
+  int dbg;  // profiling experiments: bit0 skip MFMA loop, bit1 skip column sums, bit2 skip epilogue
+};
+
+template <typename T, int KCH, bool VEC>
+__global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
+  using R = Real<T>;
+  using acc_t = typename R::acc_t;
+  constexpr int VW = R::VW;             // elements per 16-byte vector
+  constexpr int TS = 64;                // tile side
+  constexpr int G = TS / VW;            // 16-byte groups per tile row
+  constexpr int RPP = 256 / G;          // tile rows covered by the workgroup per pass
+  constexpr int PASSES = TS / RPP;      // passes over the tile (epilogue, Cij prefetch)
+  constexpr int SP = KCH / RPP;         // staging passes per chunk
+  constexpr int CP = TS + VW;           // pitch of the accumulator tile in LDS
+  static_assert(KCH % RPP == 0 && KCH % 4 == 0, "chunk size");
+  constexpr int SLAB = 2 * KCH * TS > TS * CP ? 2 * KCH * TS : TS * CP;  // staging, then accumulators
+
+  __shared__ __attribute__((aligned(16))) T slab[SLAB];  // xs | ys, later the accumulator tile
+  __shared__ T rci_s[TS], rcj_s[TS];
+  T *xs = slab, *ys = slab + KCH * TS;
+
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, p = lane & 15, q = lane >> 4;
+  const long it = (long)blockIdx.x / a.tiles_j, jt = (long)blockIdx.x % a.tiles_j;
+  const long i0 = it * TS, j0 = jt * TS;
+
+  // thread's share of the tile in row-major order: VW columns of PASSES rows
+  const int eg = tid % G, er = tid / G;
+  const long ecol = j0 + VW * eg;
+
+  // ---- 1. Cij prefetch
+  T cpre[PASSES][VW];
+#pragma unroll
+  for (int k = 0; k < PASSES; k++) {
+    const long row = i0 + er + RPP * k;
+    load_vw<T, VEC>(cpre[k], a.Cij + row * a.M, ecol, a.M, row < a.N);
+  }
+
+  // mask bits of the thread's PASSES x VW synapses, requested now for the same reason
+  uint32_t onbits = 0xffffffffu;
+  if (a.wmask) {
+    uint32_t hc[VW];
+#pragma unroll
+    for (int e = 0; e < VW; e++) hc[e] = (ecol + e < a.M) ? (uint32_t)(ecol + e) / (uint32_t)a.Mc : 0u;
+    // the VW columns usually sit in one hypercolumn: then one mask byte serves the vector
+    const bool one_hc = (ecol + VW - 1 < a.M) && hc[0] == hc[VW - 1];
+    onbits = 0;
+#pragma unroll
+    for (int k = 0; k < PASSES; k++) {
+      const long row = i0 + er + RPP * k;
+      if (row >= a.N) continue;
+      const uint8_t *mrow = a.wmask + row * a.H;
+      if (one_hc) {
+        if (mrow[hc[0]] != 0) onbits |= ((1u << VW) - 1u) << (VW * k);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VW; e++)
+          if (ecol + e < a.M && mrow[hc[e]] != 0) onbits |= 1u << (VW * k + e);
+      }
+    }
+  }
+
+  acc_t acc[2][2];
+#pragma unroll
+  for (int r = 0; r < 2; r++)
+#pragma unroll
+    for (int c = 0; c < 2; c++) acc[r][c] = acc_t{0, 0, 0, 0};
+  const int iw = (w >> 1) * 32, jw = (w & 1) * 32;  // sub-tile of this wavefront
+
+  // column sums: lanes 0..31 of wavefronts 0,1 take the 64 x columns, of wavefronts 2,3 the y columns
+  const bool summer = lane < 32;
+  const bool sum_i = w < 2;
+  const int scol = (w & 1) * 32 + (lane & 31);
+  const T *sbase = (sum_i ? xs : ys) + scol;
+  const long sidx = (sum_i ? i0 : j0) + scol;
+  const bool sum_ok = summer && sidx < (sum_i ? a.N : a.M);
+  const bool writes_bias = sum_ok && !sum_i && it == 0 && a.bias_mode == 1;
+  const T cold = sum_ok ? (sum_i ? a.Ci : a.Cj)[sidx] : T(1);  // old trace, requested early
+  T kb = writes_bias ? a.kbi[sidx] : T(1);
+  T csum = T(0);
+
+  // ---- 2./3. chunks of the batch
+  for (long b0 = 0; b0 < a.B; b0 += KCH) {
+    const long rows = a.B - b0 < KCH ? a.B - b0 : KCH;
+    if (b0 > 0) __syncthreads();  // previous chunk fully consumed
+    T sx[SP][VW], sy[SP][VW];
+#pragma unroll
+    for (int m = 0; m < SP; m++) {
+      const long b = b0 + er + RPP * m;
+      load_vw<T, VEC>(sx[m], a.x + b * a.N, i0 + VW * eg, a.N, b < a.B);
+      load_vw<T, VEC>(sy[m], a.y + b * a.M, ecol, a.M, b < a.B);
+    }
+#pragma unroll
+    for (int m = 0; m < SP; m++) {
+      typename R::vec_t vx, vy;
+#pragma unroll
+      for (int e = 0; e < VW; e++) {
+        vx[e] = sx[m][e];
+        vy[e] = sy[m][e];
+      }
+      *reinterpret_cast<typename R::vec_t *>(&xs[(er + RPP * m) * TS + VW * eg]) = vx;
+      *reinterpret_cast<typename R::vec_t *>(&ys[(er + RPP * m) * TS + VW * eg]) = vy;
+    }
+    __syncthreads();
+
+    if (summer && !(a.dbg & 2)) {
+      // rows past the end of the batch were staged as zeros: adding them changes nothing, so the loop
+      // needs no guard; 32 LDS reads are in flight before the (ordered) additions consume them
+      (void)rows;
+      for (int r = 0; r < KCH; r += 32) {
+        T v[32];
+#pragma unroll
+        for (int k = 0; k < 32; k++) v[k] = sbase[(r + k) * TS];
+#pragma unroll
+        for (int k = 0; k < 32; k++) csum = R::add(csum, v[k]);
+      }
+    }
+
+    // K loop: per step of 4 batch rows, lane (p,q) feeds row 4s+q of the slabs
+    const T *xa = xs + q * TS + iw + 2 * p;
+    const T *ya = ys + q * TS + jw + 2 * p;
+    if (!(a.dbg & 1))
+#pragma unroll 8
+    for (int s = 0; s < KCH / 4; s++) {
+      const T x0 = xa[s * 4 * TS], x1 = xa[s * 4 * TS + 1];
+      const T y0 = ya[s * 4 * TS], y1 = ya[s * 4 * TS + 1];
+      acc[0][0] = R::mfma(x0, y0, acc[0][0]);
+      acc[0][1] = R::mfma(x0, y1, acc[0][1]);
+      acc[1][0] = R::mfma(x1, y0, acc[1][0]);
+      acc[1][1] = R::mfma(x1, y1, acc[1][1]);
+    }
+  }
+
+  // ---- 3. new traces of this tile's rows and columns (reference order of operations)
+  if (summer) {
+    T cnew = T(1);
+    if (sum_ok) {
+      T s = R::div(csum, a.fB);
+      s = R::mul(s, a.tau);
+      cnew = R::add(R::mul(cold, a.omt), s);
+      cnew = cnew > T(0) ? cnew : T(0);
+      if (sum_i) {
+        if (jt == 0) a.Ci_next[sidx] = cnew;
+      } else if (it == 0) {
+        a.Cj_next[sidx] = cnew;
+        if (writes_bias) {
+          a.bias[sidx] = bias_regularized<T>(cnew, kb, a.cthr, a.khalf, a.pmin, a.taubdt);
+          a.kbi[sidx] = kb;
+        }
+      }
+    }
+    (sum_i ? rci_s : rcj_s)[scol] = trace_reciprocal<T>(cnew, a.cthr);
+  }
+  __syncthreads();  // slabs consumed, reciprocals published
+
+  if (a.dbg & 4) {
+    if (acc[0][0][0] == T(12345.678)) a.W[0] = acc[0][0][0] + cpre[0][0];
+    return;
+  }
+  // ---- 4. accumulators -> row-major LDS tile
+  T *cs = slab;
+#pragma unroll
+  for (int r = 0; r < 2; r++)
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+      const int row = iw + 2 * R::acc_row(q, v) + r;
+      cs[row * CP + jw + 2 * p] = acc[r][0][v];
+      cs[row * CP + jw + 2 * p + 1] = acc[r][1][v];
+    }
+  __syncthreads();
+
+  // ---- epilogue: decay + clamp, weight, mask, stores
+  T rcj[VW];
+#pragma unroll
+  for (int e = 0; e < VW; e++) rcj[e] = rcj_s[VW * eg + e];
+#pragma unroll
+  for (int k = 0; k < PASSES; k++) {
+    const int lr = er + RPP * k;
+    const long row = i0 + lr;
+    if (row >= a.N) continue;
+    const T rci = rci_s[lr];
+    T cv[VW], wv[VW];
+#pragma unroll
+    for (int e = 0; e < VW; e++) {
+      T t = cs[lr * CP + VW * eg + e] * a.invB;
+      t = t * a.tau;
+      T cn = cpre[k][e] * a.omt + t;
+      cn = cn > T(0) ? cn : T(0);
+      cv[e] = cn;
+      const T wgt = weight_from_traces<T>(cn, rci, rcj[e], a.cthr4);
+      wv[e] = ((onbits >> (VW * k + e)) & 1u) ? wgt : T(0);
+    }
+    store_vw<T, VEC>(cv, a.Cij + row * a.M, ecol, a.M);
+    store_vw<T, VEC>(wv, a.W + row * a.M, ecol, a.M);
+  }
+}
+
+}  // namespace sb

@@ -7,156 +7,6 @@
 
 namespace sb {
 
-// =====================================================================================================
-// Forward: act = softmax_per_hypercolumn(x . W + bias)            omp.cc:70-87 + kernels_numpy.py:13-25
-//
-// A workgroup of 4 wavefronts owns 16 batch rows x one column tile (one whole hypercolumn when FUSE,
-// NG*16*VW arbitrary columns otherwise).  The 4 wavefronts split the reduction dimension N in
-// interleaved chunks of 4*VW; each runs 16x16x4 MFMAs with
-//   A = x   : lane (p,q) loads VW consecutive k of batch row b0+p      -> VW MFMA steps
-//   B = W   : lane (p,q) loads VW consecutive columns of W row k       -> VW column blocks
-// so one 16-byte load of x and VW*NG 16-byte loads of W feed VW*VW*NG MFMAs.  Column block c of
-// group g holds columns j0 + g*16*VW + VW*p + c (interleaved), which makes every result vector
-// {c = 0..VW-1} VW consecutive columns.  Partial tiles are summed through LDS in a fixed order
-// ((w0+w2)+(w1+w3)), then 16 threads per row add the bias and, when FUSE, do the softmax.
-// =====================================================================================================
-template <typename T>
-struct ForwardArgs {
-  T *act;
-  const T *x;
-  const T *W;
-  const T *bias;
-  long B, N, M, Mc;
-};
-
-template <typename T, int NG, bool FUSE, bool VEC>
-__global__ __launch_bounds__(256) void k_forward(ForwardArgs<T> a) {
-  constexpr int VW = Real<T>::VW;
-  constexpr int GW = 16 * VW;
-  constexpr int CP = NG * GW + VW;
-  using acc_t = typename Real<T>::acc_t;
-  using vec_t = typename Real<T>::vec_t;
-  __shared__ __attribute__((aligned(16))) T red[2][16][CP];
-
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, p = lane & 15, q = lane >> 4;
-  const long b0 = (long)blockIdx.y * 16;
-  const long j0 = FUSE ? (long)blockIdx.x * a.Mc : (long)blockIdx.x * (NG * GW);
-  const long jend = FUSE ? j0 + a.Mc : (j0 + NG * GW < a.M ? j0 + NG * GW : a.M);
-  const long nchunks = (a.N + 4 * VW - 1) / (4 * VW);
-  const bool row_ok = (b0 + p) < a.B;
-  const T *xrow = a.x + (b0 + p) * a.N;
-
-  acc_t acc[NG][VW];
-#pragma unroll
-  for (int g = 0; g < NG; g++)
-#pragma unroll
-    for (int c = 0; c < VW; c++) acc[g][c] = acc_t{0, 0, 0, 0};
-
-  T xa[VW], xb[VW];
-  T wa[VW][NG][VW], wb[VW][NG][VW];
-
-  auto load_chunk = [&](long kc, T(&xo)[VW], T(&wo)[VW][NG][VW]) {
-    const long kk = kc * (4 * VW) + VW * q;
-    const bool ok = kc < nchunks;
-    load_vw<T, VEC>(xo, xrow, kk, a.N, row_ok && ok);
-#pragma unroll
-    for (int s = 0; s < VW; s++) {
-      const long krow = kk + s;
-      const bool kok = ok && krow < a.N;
-      const T *wrow = a.W + krow * a.M;
-#pragma unroll
-      for (int g = 0; g < NG; g++) load_vw<T, VEC>(wo[s][g], wrow, j0 + g * GW + VW * p, jend, kok);
-    }
-  };
-  auto compute = [&](const T(&xi)[VW], const T(&wi)[VW][NG][VW]) {
-#pragma unroll
-    for (int s = 0; s < VW; s++)
-#pragma unroll
-      for (int g = 0; g < NG; g++)
-#pragma unroll
-        for (int c = 0; c < VW; c++) acc[g][c] = Real<T>::mfma(xi[s], wi[s][g][c], acc[g][c]);
-  };
-
-  load_chunk(w, xa, wa);
-  for (long kc = w; kc < nchunks; kc += 8) {
-    load_chunk(kc + 4, xb, wb);
-    compute(xa, wa);
-    load_chunk(kc + 8, xa, wa);
-    compute(xb, wb);
-  }
-
-  // ---- cross-wavefront sum through LDS: slots 0/1 end up holding (w0+w2) and (w1+w3)
-  if (w >= 2) {
-#pragma unroll
-    for (int g = 0; g < NG; g++)
-#pragma unroll
-      for (int v = 0; v < 4; v++) {
-        vec_t t;
-#pragma unroll
-        for (int c = 0; c < VW; c++) t[c] = acc[g][c][v];
-        *reinterpret_cast<vec_t *>(&red[w - 2][Real<T>::acc_row(q, v)][g * GW + VW * p]) = t;
-      }
-  }
-  __syncthreads();
-  if (w < 2) {
-#pragma unroll
-    for (int g = 0; g < NG; g++)
-#pragma unroll
-      for (int v = 0; v < 4; v++) {
-        vec_t *slot = reinterpret_cast<vec_t *>(&red[w][Real<T>::acc_row(q, v)][g * GW + VW * p]);
-        vec_t t = *slot;
-#pragma unroll
-        for (int c = 0; c < VW; c++) t[c] = acc[g][c][v] + t[c];
-        *slot = t;
-      }
-  }
-  __syncthreads();
-
-  // ---- bias (+ softmax): 16 threads per batch row, thread handles columns l16, l16+16, ...
-  const int row = tid >> 4, l16 = tid & 15;
-  const long ncol = jend - j0;
-  constexpr int PER = NG * VW;
-  T vals[PER];
-  T mx = -INFINITY;
-#pragma unroll
-  for (int t = 0; t < PER; t++) {
-    const long col = l16 + 16 * t;
-    vals[t] = T(0);
-    if (col < ncol) {
-      vals[t] = (red[0][row][col] + red[1][row][col]) + a.bias[j0 + col];
-      mx = vals[t] > mx ? vals[t] : mx;
-    }
-  }
-  if (FUSE) {
-#pragma unroll
-    for (int o = 8; o >= 1; o >>= 1) {
-      const T other = __shfl_xor(mx, o);
-      mx = other > mx ? other : mx;
-    }
-    T sum = T(0);
-#pragma unroll
-    for (int t = 0; t < PER; t++) {
-      const long col = l16 + 16 * t;
-      if (col < ncol) {
-        vals[t] = Real<T>::exp_(vals[t] - mx);
-        sum += vals[t];
-      }
-    }
-#pragma unroll
-    for (int o = 8; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
-#pragma unroll
-    for (int t = 0; t < PER; t++) vals[t] = vals[t] / sum;
-  }
-  if (b0 + row < a.B) {
-    T *out = a.act + (b0 + row) * a.M + j0;
-#pragma unroll
-    for (int t = 0; t < PER; t++) {
-      const long col = l16 + 16 * t;
-      if (col < ncol) out[col] = vals[t];
-    }
-  }
-}
-
 // Softmax over each (row, hypercolumn) group of Mc values, in place; one wavefront per group.
 // kernels_numpy.py:13-25
 template <typename T>
@@ -213,30 +63,6 @@ __device__ __forceinline__ T bias_regularized(T pj, T &kbi, T cthr, T khalf, T p
   return (pj < cthr) ? R::mul(kbi, R::log_(R::mul(T(2), cthr))) : R::mul(kbi, R::log_(pj));
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void k_counters(CountersArgs<T> a) {
-  using R = Real<T>;
-  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
-  const bool is_i = idx < a.N;
-  const long col = is_i ? idx : idx - a.N;
-  const long ld = is_i ? a.N : a.M;
-  if (!is_i && col >= a.M) return;
-  const T *src = (is_i ? a.x : a.y) + col;
-  T s = T(0);
-  for (long b = 0; b < a.B; b++) s = R::add(s, src[b * ld]);
-  s = R::div(s, a.fB);
-  s = R::mul(s, a.tau);
-  T *C = is_i ? a.Ci : a.Cj;
-  T c = R::add(R::mul(C[col], a.omt), s);
-  c = c > T(0) ? c : T(0);
-  C[col] = c;
-  if (!is_i && a.bias_mode == 1) {
-    T kb = a.kbi[col];
-    a.bias[col] = bias_regularized<T>(c, kb, a.cthr, a.khalf, a.pmin, a.taubdt);
-    a.kbi[col] = kb;
-  }
-}
-
 // omp.cc:207-220
 template <typename T>
 __global__ __launch_bounds__(256) void k_update_bias(T *bias, const T *Cj, T cthr, long M) {
@@ -255,168 +81,6 @@ __global__ __launch_bounds__(256) void k_update_bias_regularized(T *bias, T *kbi
   T kb = kbi[j];
   bias[j] = bias_regularized<T>(Cj[j], kb, cthr, khalf, pmin, taubdt);
   kbi[j] = kb;
-}
-
-// =====================================================================================================
-// Cij moving average as a rank-B MFMA update with the decay, clamp, weight recompute and mask apply in
-// the epilogue:                                                          omp.cc:158-201, 322-335
-//   Cij <- max(0, Cij*(1-taupdt) + (x^T y / B) * taupdt)
-//   W   <- wmask ? log(max(Cij, cthr^4) / (Ci*Cj)) : 0     (0 as well where Ci < cthr or Cj < cthr)
-// Ci and Cj are this step's already-updated traces.
-//
-// A wavefront owns a (RX*16*VW) x (RY*16*VW) tile of Cij for the whole batch (K = B).  Both operands
-// are "k-major" in memory (x[b][i], y[b][j]), exactly the MFMA operand layout, so they are loaded
-// straight from L2 into registers: lane (p,q) loads VW consecutive i (resp. j) of batch row 4s+q.
-// Block (r,c) of the tile then holds rows i0 + VW*p16 + r and columns j0 + VW*p + c, which turns every
-// Cij / W access of the epilogue into one 16-byte vector per lane (256 contiguous bytes per 16 lanes).
-// With PRE the Cij tile is requested before the K loop so HBM latency hides behind the MFMAs.
-// =====================================================================================================
-template <typename T>
-struct TraceArgs {
-  const T *x;  // [B,N]
-  const T *y;  // [B,M]
-  T *Cij;
-  T *W;
-  const T *Ci;
-  const T *Cj;
-  const uint8_t *wmask;  // [N,H] or nullptr (no mask: every synapse active)
-  long B, N, M, H, Mc;
-  T tau, omt, invB, cthr, cthr4;
-};
-
-template <typename T, int RX, int RY, bool VEC, bool PRE>
-__global__ __launch_bounds__(256) void k_trace_weights(TraceArgs<T> a) {
-  constexpr int VW = Real<T>::VW;
-  constexpr int GW = 16 * VW;
-  constexpr int TI = RX * GW, TJ = RY * GW;
-  using acc_t = typename Real<T>::acc_t;
-
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, p = lane & 15, q = lane >> 4;
-  const long i0 = ((long)blockIdx.y * 2 + (w >> 1)) * TI;
-  const long j0 = ((long)blockIdx.x * 2 + (w & 1)) * TJ;
-  if (i0 >= a.N || j0 >= a.M) return;  // wavefront-uniform; the kernel has no barriers
-
-  T cpre[PRE ? RX : 1][VW][4][PRE ? RY : 1][VW];
-  if (PRE) {
-#pragma unroll
-    for (int rx = 0; rx < RX; rx++)
-#pragma unroll
-      for (int r = 0; r < VW; r++)
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-          const long row = i0 + rx * GW + VW * Real<T>::acc_row(q, v) + r;
-#pragma unroll
-          for (int ry = 0; ry < RY; ry++)
-            load_vw<T, VEC>(cpre[rx][r][v][ry], a.Cij + row * a.M, j0 + ry * GW + VW * p, a.M,
-                            row < a.N);
-        }
-  }
-
-  acc_t acc[RX * VW][RY * VW];
-#pragma unroll
-  for (int i = 0; i < RX * VW; i++)
-#pragma unroll
-    for (int j = 0; j < RY * VW; j++) acc[i][j] = acc_t{0, 0, 0, 0};
-
-  constexpr int PF = 4;
-  T xr[PF][RX][VW], yr[PF][RY][VW];
-  auto load_step = [&](long s, T(&xo)[RX][VW], T(&yo)[RY][VW]) {
-    const long b = 4 * s + q;
-    const bool ok = b < a.B;
-    const T *xrow = a.x + b * a.N;
-    const T *yrow = a.y + b * a.M;
-#pragma unroll
-    for (int rx = 0; rx < RX; rx++) load_vw<T, VEC>(xo[rx], xrow, i0 + rx * GW + VW * p, a.N, ok);
-#pragma unroll
-    for (int ry = 0; ry < RY; ry++) load_vw<T, VEC>(yo[ry], yrow, j0 + ry * GW + VW * p, a.M, ok);
-  };
-#pragma unroll
-  for (int u = 0; u < PF; u++) load_step(u, xr[u], yr[u]);
-  const long nsteps = (a.B + 3) / 4;
-  for (long s0 = 0; s0 < nsteps; s0 += PF) {
-#pragma unroll
-    for (int u = 0; u < PF; u++) {
-      T xa[RX][VW], ya[RY][VW];
-#pragma unroll
-      for (int rx = 0; rx < RX; rx++)
-#pragma unroll
-        for (int e = 0; e < VW; e++) xa[rx][e] = xr[u][rx][e];
-#pragma unroll
-      for (int ry = 0; ry < RY; ry++)
-#pragma unroll
-        for (int e = 0; e < VW; e++) ya[ry][e] = yr[u][ry][e];
-      load_step(s0 + u + PF, xr[u], yr[u]);
-#pragma unroll
-      for (int rx = 0; rx < RX; rx++)
-#pragma unroll
-        for (int r = 0; r < VW; r++)
-#pragma unroll
-          for (int ry = 0; ry < RY; ry++)
-#pragma unroll
-            for (int c = 0; c < VW; c++)
-              acc[rx * VW + r][ry * VW + c] =
-                  Real<T>::mfma(xa[rx][r], ya[ry][c], acc[rx * VW + r][ry * VW + c]);
-    }
-  }
-
-  // ---- epilogue
-  T rci_l[RX][VW], rcj_l[RY][VW];
-  uint32_t hc_l[RY][VW];
-#pragma unroll
-  for (int rx = 0; rx < RX; rx++)
-#pragma unroll
-    for (int r = 0; r < VW; r++) {
-      const long row = i0 + rx * GW + VW * p + r;
-      rci_l[rx][r] = trace_reciprocal<T>(row < a.N ? a.Ci[row] : T(1), a.cthr);
-    }
-#pragma unroll
-  for (int ry = 0; ry < RY; ry++)
-#pragma unroll
-    for (int c = 0; c < VW; c++) {
-      const long col = j0 + ry * GW + VW * p + c;
-      rcj_l[ry][c] = trace_reciprocal<T>(col < a.M ? a.Cj[col] : T(1), a.cthr);
-      hc_l[ry][c] = col < a.M ? (uint32_t)col / (uint32_t)a.Mc : 0u;
-    }
-
-#pragma unroll
-  for (int rx = 0; rx < RX; rx++)
-#pragma unroll
-    for (int r = 0; r < VW; r++)
-#pragma unroll
-      for (int v = 0; v < 4; v++) {
-        const int p16 = Real<T>::acc_row(q, v);
-        const long row = i0 + rx * GW + VW * p16 + r;
-        const T rci = __shfl(rci_l[rx][r], p16);
-        if (row < a.N) {
-          T *crow = a.Cij + row * a.M;
-          T *wrow = a.W + row * a.M;
-          const uint8_t *mrow = a.wmask ? a.wmask + row * a.H : nullptr;
-#pragma unroll
-          for (int ry = 0; ry < RY; ry++) {
-            const long col = j0 + ry * GW + VW * p;
-            T cv[VW], wv[VW];
-            if (PRE) {
-#pragma unroll
-              for (int c = 0; c < VW; c++) cv[c] = cpre[rx][r][v][ry][c];
-            } else {
-              load_vw<T, VEC>(cv, crow, col, a.M, true);
-            }
-#pragma unroll
-            for (int c = 0; c < VW; c++) {
-              T t = acc[rx * VW + r][ry * VW + c][v] * a.invB;
-              t = t * a.tau;
-              T cn = cv[c] * a.omt + t;
-              cn = cn > T(0) ? cn : T(0);
-              cv[c] = cn;
-              T wgt = weight_from_traces<T>(cn, rci, rcj_l[ry][c], a.cthr4);
-              if (mrow && col + c < a.M && mrow[hc_l[ry][c]] == 0) wgt = T(0);
-              wv[c] = wgt;
-            }
-            store_vw<T, VEC>(cv, crow, col, a.M);
-            store_vw<T, VEC>(wv, wrow, col, a.M);
-          }
-        }
-      }
 }
 
 // omp.cc:322-335
@@ -666,3 +330,7 @@ __global__ __launch_bounds__(256) void k_fill(T *dst, T value, size_t n) {
 }
 
 }  // namespace sb
+
+#include "sb_k_forward.hpp"
+#include "sb_k_traces.hpp"
+#include "sb_k_mask_swap.hpp"

@@ -31,7 +31,7 @@ struct TraceScalars {
 // with a pair of HIP events on the launch stream; sb_profile_stop sums the elapsed times per kernel.
 enum KernelId {
   K_FORWARD = 0, K_SOFTMAX, K_COUNTERS, K_TRACE_WEIGHTS, K_UPDATE_BIAS, K_UPDATE_BIAS_REG, K_MASK_SCORES,
-  K_MASK_SWAP, K_MASK_FIX, K_APPLY_MASK, K_ARGMAX, K_GATHER, K_FILL, K_COUNT
+  K_MASK_SWAP, K_MASK_FIX, K_APPLY_MASK, K_ARGMAX, K_GATHER, K_FILL, K_TRAIN_FUSED, K_COUNT
 };
 const char *kernel_name(int id);
 struct ProfScope {
@@ -58,9 +58,18 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
     }                                                 \
   } while (0)
 
+// The split-K forward needs scratch for its partial sums: forward_plan says how many elements (0 when
+// the shape does not qualify); launch_forward uses that path when `scratch` is large enough and falls
+// back to the single-kernel forms otherwise.
+struct ForwardPlan {
+  long KS;             // slices of the reduction dimension
+  long scratch_elems;  // KS * B * M, or 0
+};
+template <typename T>
+ForwardPlan forward_plan(long B, long N, long H, long Mc);
 template <typename T>
 int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias, long B, long N,
-                   long H, long Mc, bool softmax);
+                   long H, long Mc, bool softmax, T *scratch, size_t scratch_elems);
 template <typename T>
 int launch_softmax(hipStream_t st, T *act, long B, long H, long Mc);
 template <typename T>
@@ -70,6 +79,12 @@ template <typename T>
 int launch_trace_weights(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci,
                          const T *Cj, const uint8_t *wmask, long B, long N, long H, long Mc, T taupdt,
                          T cthr);
+// Fused Ci/Cj/Cij + weights (+ regularised bias when bias_mode == 1, + mask when wmask != nullptr).
+// Reads the old traces from Ci/Cj and writes the new ones to Ci_next/Cj_next (distinct buffers).
+template <typename T>
+int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci, const T *Cj,
+                       T *Ci_next, T *Cj_next, const uint8_t *wmask, int bias_mode, T *bias, T *kbi,
+                       long B, long N, long H, long Mc, T taupdt, T cthr, T khalf, T pmin, T taubdt);
 template <typename T>
 int launch_update_bias(hipStream_t st, T *bias, const T *Cj, T cthr, long M);
 template <typename T>

@@ -2,7 +2,11 @@
 // sb_kernels_f32.hip / sb_kernels_f64.hip, which instantiate them explicitly.
 #pragma once
 #include "sb_kernels.hpp"
+#include "sb_k_train.hpp"
+#include "sb_k_forward_splitk.hpp"
 #include "sb_launch.hpp"
+
+#include <cstdlib>
 
 namespace sb {
 
@@ -13,43 +17,130 @@ static inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 
 // ------------------------------------------------------------------------------------------- forward
 template <typename T, int NG, bool FUSE>
-static int forward_variant(hipStream_t st, const ForwardArgs<T> &a, dim3 grid, bool vec) {
+static int forward_variant(hipStream_t st, ForwardArgs<T> a, bool vec) {
   ProfScope prof_(st, K_FORWARD);
+  // 8 workgroup ids per round of XCDs; ids beyond the last tile exit at once
+  const long ntiles = a.col_tiles * a.batch_tiles;
+  const long grid = 8 * cdiv(ntiles, 8);
+  if (grid >= (1L << 31)) {
+    set_error("launch_forward: too many tiles for one launch");
+    return -1;
+  }
+  static const int waves_env = [] {
+    const char *e = getenv("SB_FWD_WAVES");
+    return e ? atoi(e) : 0;
+  }();
+  if constexpr (NG <= 2) {
+    if (waves_env == 16) {
+      if (vec)
+        hipLaunchKernelGGL((k_forward<T, NG, FUSE, true, 16>), dim3((unsigned)grid), dim3(1024), 0, st, a);
+      else
+        hipLaunchKernelGGL((k_forward<T, NG, FUSE, false, 16>), dim3((unsigned)grid), dim3(1024), 0, st, a);
+      SB_LAUNCH_CHECK();
+      return 0;
+    }
+  }
   if (vec)
-    hipLaunchKernelGGL((k_forward<T, NG, FUSE, true>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((k_forward<T, NG, FUSE, true, 8>), dim3((unsigned)grid), dim3(512), 0, st, a);
   else
-    hipLaunchKernelGGL((k_forward<T, NG, FUSE, false>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((k_forward<T, NG, FUSE, false, 8>), dim3((unsigned)grid), dim3(512), 0, st, a);
   SB_LAUNCH_CHECK();
   return 0;
 }
 
+static inline int device_cu_count() {
+  static const int n = [] {
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) {
+      hipDeviceProp_t prop;
+      if (hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+    }
+    return cus;
+  }();
+  return n;
+}
+
+template <typename T>
+ForwardPlan forward_plan(long B, long N, long H, long Mc) {
+  constexpr int VW = Real<T>::VW;
+  ForwardPlan plan{0, 0};
+  if (cdiv(Mc, 16 * VW) > 8 || B <= 0 || N <= 0 || H <= 0) return plan;
+  const long chunks = cdiv(N, 4 * VW);
+  const long tiles = cdiv(B, 128) * H;
+  long ks = device_cu_count() / tiles;  // about one workgroup per CU
+  static const int ks_env = [] {
+    const char *e = getenv("SB_FWD_KS");
+    return e ? atoi(e) : 0;
+  }();
+  if (ks_env > 0) ks = ks_env;
+  if (ks < 1) ks = 1;
+  if (ks > chunks) ks = chunks;
+  plan.KS = ks;
+  plan.scratch_elems = ks * B * H * Mc;
+  return plan;
+}
+
 template <typename T>
 int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias, long B, long N,
-                   long H, long Mc, bool softmax) {
+                   long H, long Mc, bool softmax, T *scratch, size_t scratch_elems) {
   constexpr int VW = Real<T>::VW;
   constexpr int GW = 16 * VW;
   SB_REQUIRE(act && x && W && bias, "null pointer");
   SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");
   const long M = H * Mc;
   SB_REQUIRE(M < (1L << 31) && N < (1L << 31), "dimension too large");
-  SB_REQUIRE(cdiv(B, 16) <= 65535, "batch too large for one launch");
-  ForwardArgs<T> a{act, x, W, bias, B, N, M, Mc};
+  ForwardArgs<T> a{act, x, W, bias, B, N, M, Mc, 0, cdiv(B, 16), 0};
+  {
+    const char *e = getenv("SB_DBG");
+    a.dbg = e ? atoi(e) : 0;
+  }
   const bool base_vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(W);
   const long need = cdiv(Mc, GW);
+  // split-K path: needs the partial-sum scratch and a hypercolumn that fits one staged tile
+  const ForwardPlan plan = forward_plan<T>(B, N, H, Mc);
+  // measured slower than the single-kernel form at the MNIST shape (two launches, partial-sum round
+  // trip); kept selectable for shapes with many batch rows per hypercolumn
+  static const bool no_splitk = getenv("SB_FWD_SPLIT") == nullptr;
+  if (softmax && plan.scratch_elems > 0 && scratch && scratch_elems >= (size_t)plan.scratch_elems &&
+      !no_splitk) {
+    ForwardSplitArgs<T> sa{scratch, x, W, B, N, M, H, Mc, plan.KS, cdiv(N, 4 * VW), a.dbg};
+    const bool vec = base_vec && (Mc % VW == 0) && aligned16(scratch);
+    const long grid = cdiv(B, 128) * H * plan.KS;
+    SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
+    {
+      ProfScope prof_(st, K_FORWARD);
+#define SB_FWD_SPLIT(NG_)                                                                            \
+  do {                                                                                               \
+    if (vec)                                                                                         \
+      hipLaunchKernelGGL((k_forward_splitk<T, NG_, true>), dim3((unsigned)grid), dim3(512), 0, st, sa); \
+    else                                                                                             \
+      hipLaunchKernelGGL((k_forward_splitk<T, NG_, false>), dim3((unsigned)grid), dim3(512), 0, st, sa); \
+  } while (0)
+      if (need <= 1) SB_FWD_SPLIT(1);
+      else if (need <= 2) SB_FWD_SPLIT(2);
+      else if (need <= 4) SB_FWD_SPLIT(4);
+      else SB_FWD_SPLIT(8);
+#undef SB_FWD_SPLIT
+      SB_LAUNCH_CHECK();
+    }
+    ProfScope prof_(st, K_SOFTMAX);
+    hipLaunchKernelGGL((k_forward_finish<T>), dim3((unsigned)cdiv(B * H, 4)), dim3(256), 0, st, act,
+                       (const T *)scratch, bias, B, M, H, Mc, plan.KS, 1);
+    SB_LAUNCH_CHECK();
+    return 0;
+  }
   const long max_fused = sizeof(T) == 4 ? 4 : 7;
   if (softmax && need <= max_fused) {
     const bool vec = base_vec && (Mc % VW == 0);
-    dim3 grid((unsigned)H, (unsigned)cdiv(B, 16));
-    if (need <= 1) return forward_variant<T, 1, true>(st, a, grid, vec);
-    if (need <= 2) return forward_variant<T, 2, true>(st, a, grid, vec);
-    if (need <= 4) return forward_variant<T, 4, true>(st, a, grid, vec);
-    if constexpr (sizeof(T) == 8) return forward_variant<T, 7, true>(st, a, grid, vec);
+    a.col_tiles = H;
+    if (need <= 1) return forward_variant<T, 1, true>(st, a, vec);
+    if (need <= 2) return forward_variant<T, 2, true>(st, a, vec);
+    if (need <= 4) return forward_variant<T, 4, true>(st, a, vec);
+    if constexpr (sizeof(T) == 8) return forward_variant<T, 7, true>(st, a, vec);
   }
-  {
-    dim3 grid((unsigned)cdiv(M, 2 * GW), (unsigned)cdiv(B, 16));
-    int rc = forward_variant<T, 2, false>(st, a, grid, base_vec);
-    if (rc) return rc;
-  }
+  a.col_tiles = cdiv(M, 2 * GW);
+  int rc = forward_variant<T, 2, false>(st, a, base_vec);
+  if (rc) return rc;
   if (softmax) return launch_softmax<T>(st, act, B, H, Mc);
   return 0;
 }
@@ -80,27 +171,42 @@ int launch_counters(hipStream_t st, const T *x, const T *y, T *Ci, T *Cj, long B
   a.bias_mode = bias_mode; a.bias = bias; a.kbi = kbi;
   a.cthr = cthr; a.khalf = khalf; a.pmin = pmin; a.taubdt = taubdt;
   ProfScope prof_(st, K_COUNTERS);
-  hipLaunchKernelGGL((k_counters<T>), dim3((unsigned)cdiv(N + M, 256)), dim3(256), 0, st, a);
+  hipLaunchKernelGGL((k_counters<T>), dim3((unsigned)(cdiv(N, 64) + cdiv(M, 64))), dim3(256), 0, st, a);
   SB_LAUNCH_CHECK();
   return 0;
 }
 
 // ------------------------------------------------------------------------------------- trace + weights
-template <typename T, int RX, int RY>
+template <typename T, int XW, int YW, int RX, int RY>
 static int trace_variant(hipStream_t st, const TraceArgs<T> &a, bool vec) {
-  constexpr int GW = 16 * Real<T>::VW;
-  dim3 grid((unsigned)cdiv(a.M, 2 * RY * GW), (unsigned)cdiv(a.N, 2 * RX * GW));
+  ProfScope prof_(st, K_TRACE_WEIGHTS);
+  dim3 grid((unsigned)cdiv(a.M, 2 * RY * 16 * YW), (unsigned)cdiv(a.N, 2 * RX * 16 * XW));
   if (grid.y > 65535) {
     set_error("launch_trace_weights: in_features too large for one launch");
     return -1;
   }
-  ProfScope prof_(st, K_TRACE_WEIGHTS);
   if (vec)
-    hipLaunchKernelGGL((k_trace_weights<T, RX, RY, true, true>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((k_trace_weights<T, XW, YW, RX, RY, true, true>), grid, dim3(256), 0, st, a);
   else
-    hipLaunchKernelGGL((k_trace_weights<T, RX, RY, false, true>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((k_trace_weights<T, XW, YW, RX, RY, false, true>), grid, dim3(256), 0, st, a);
   SB_LAUNCH_CHECK();
   return 0;
+}
+
+static inline int dbg_flags() {
+  static const int v = [] {
+    const char *e = getenv("SB_DBG");
+    return e ? atoi(e) : 0;
+  }();
+  return v;
+}
+
+static inline int trace_tile_choice() {
+  static const int v = [] {
+    const char *e = getenv("SB_TRACE_TILE");
+    return e ? atoi(e) : 0;
+  }();
+  return v;
 }
 
 template <typename T>
@@ -117,12 +223,57 @@ int launch_trace_weights(hipStream_t st, const T *x, const T *y, T *Cij, T *W, c
   a.x = x; a.y = y; a.Cij = Cij; a.W = W; a.Ci = Ci; a.Cj = Cj; a.wmask = wmask;
   a.B = B; a.N = N; a.M = M; a.H = H; a.Mc = Mc;
   a.tau = s.tau; a.omt = s.omt; a.invB = (T)1 / (T)B; a.cthr = s.cthr; a.cthr4 = s.cthr4;
+  a.dbg = dbg_flags();
   const bool vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(y) && aligned16(Cij) &&
                    aligned16(W);
-  if constexpr (sizeof(T) == 4)
-    return trace_variant<T, 1, 1>(st, a, vec);
+  if constexpr (sizeof(T) == 4) {
+    switch (trace_tile_choice()) {
+      case 1: return trace_variant<T, 2, 4, 1, 1>(st, a, vec);   // 32 x 64
+      case 2: return trace_variant<T, 2, 2, 1, 1>(st, a, vec);   // 32 x 32
+      case 3: return trace_variant<T, 1, 4, 1, 1>(st, a, vec);   // 16 x 64
+      case 4: return trace_variant<T, 4, 2, 1, 1>(st, a, vec);   // 64 x 32
+      case 5: return trace_variant<T, 1, 4, 2, 1>(st, a, vec);   // 32 x 64, x as two 4-byte loads
+      default: return trace_variant<T, 4, 4, 1, 1>(st, a, vec);  // 64 x 64
+    }
+  } else {
+    return trace_variant<T, 2, 2, 1, 2>(st, a, vec);  // 32 x 64
+  }
+}
+
+// ------------------------------------------------------------------------------------- fused training
+template <typename T>
+int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci, const T *Cj,
+                       T *Ci_next, T *Cj_next, const uint8_t *wmask, int bias_mode, T *bias, T *kbi,
+                       long B, long N, long H, long Mc, T taupdt, T cthr, T khalf, T pmin, T taubdt) {
+  constexpr int VW = Real<T>::VW;
+  SB_REQUIRE(x && y && Cij && W && Ci && Cj && Ci_next && Cj_next, "null pointer");
+  SB_REQUIRE(Ci != Ci_next && Cj != Cj_next, "old and new traces must be distinct buffers");
+  SB_REQUIRE(bias_mode == 0 || (bias && kbi), "bias update needs bias and kbi");
+  SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");
+  const long M = H * Mc;
+  SB_REQUIRE(M < (1L << 31) && N < (1L << 31), "dimension too large");
+  const TraceScalars<T> s = TraceScalars<T>::from(taupdt, cthr);
+  TrainArgs<T> a;
+  a.x = x; a.y = y; a.Cij = Cij; a.W = W; a.Ci = Ci; a.Cj = Cj; a.Ci_next = Ci_next; a.Cj_next = Cj_next;
+  a.wmask = wmask; a.bias_mode = bias_mode; a.bias = bias; a.kbi = kbi;
+  a.B = B; a.N = N; a.M = M; a.H = H; a.Mc = Mc;
+  a.tau = s.tau; a.omt = s.omt; a.fB = (T)B; a.invB = (T)1 / (T)B; a.cthr = s.cthr; a.cthr4 = s.cthr4;
+  a.khalf = khalf; a.pmin = pmin; a.taubdt = taubdt;
+  a.tiles_i = cdiv(N, 64); a.tiles_j = cdiv(M, 64);
+  a.dbg = dbg_flags();
+  SB_REQUIRE(a.tiles_i * a.tiles_j < (1L << 31), "too many tiles for one launch");
+  const bool vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(y) && aligned16(Cij) &&
+                   aligned16(W);
+  const dim3 grid((unsigned)(a.tiles_i * a.tiles_j));
+  // batch rows staged per chunk: 32 KiB of LDS per workgroup, so four workgroups share a CU
+  constexpr int KCH = sizeof(T) == 4 ? 64 : 32;
+  ProfScope prof_(st, K_TRAIN_FUSED);
+  if (vec)
+    hipLaunchKernelGGL((k_train_fused<T, KCH, true>), grid, dim3(256), 0, st, a);
   else
-    return trace_variant<T, 1, 2>(st, a, vec);
+    hipLaunchKernelGGL((k_train_fused<T, KCH, false>), grid, dim3(256), 0, st, a);
+  SB_LAUNCH_CHECK();
+  return 0;
 }
 
 // ---------------------------------------------------------------------------------------------- bias
@@ -171,7 +322,12 @@ int launch_update_mask(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, 
   }
   if (iterations > 0) {
     ProfScope prof_(st, K_MASK_SWAP);
-    hipLaunchKernelGGL((k_mask_swap<T>), dim3(1), dim3(1024), 0, st, a);
+    if (N <= 2048)
+      hipLaunchKernelGGL((k_mask_swap_reg<T, 256, 8>), dim3(1), dim3(256), 0, st, a);
+    else if (N <= 8192)
+      hipLaunchKernelGGL((k_mask_swap_reg<T, 256, 32>), dim3(1), dim3(256), 0, st, a);
+    else
+      hipLaunchKernelGGL((k_mask_swap<T>), dim3(1), dim3(1024), 0, st, a);
     SB_LAUNCH_CHECK();
   }
   return 0;
@@ -241,13 +397,17 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
 }
 
 #define SB_INSTANTIATE_LAUNCHERS(T)                                                                   \
+  template ForwardPlan forward_plan<T>(long, long, long, long);                                       \
   template int launch_forward<T>(hipStream_t, T *, const T *, const T *, const T *, long, long, long, \
-                                 long, bool);                                                         \
+                                 long, bool, T *, size_t);                                            \
   template int launch_softmax<T>(hipStream_t, T *, long, long, long);                                 \
   template int launch_counters<T>(hipStream_t, const T *, const T *, T *, T *, long, long, long, T,   \
                                   int, T *, T *, T, T, T, T);                                         \
   template int launch_trace_weights<T>(hipStream_t, const T *, const T *, T *, T *, const T *,        \
                                        const T *, const uint8_t *, long, long, long, long, T, T);     \
+  template int launch_train_fused<T>(hipStream_t, const T *, const T *, T *, T *, const T *, const T *, \
+                                     T *, T *, const uint8_t *, int, T *, T *, long, long, long, long, \
+                                     T, T, T, T, T);                                                   \
   template int launch_update_bias<T>(hipStream_t, T *, const T *, T, long);                           \
   template int launch_update_bias_regularized<T>(hipStream_t, T *, T *, const T *, T, T, T, T, long); \
   template int launch_update_mask<T>(hipStream_t, uint8_t *, const T *, const T *, const T *,         \

@@ -2,7 +2,9 @@
 // device-resident network object.  Host code only; kernels live in sb_kernels.hpp.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
 #include <cstring>
+#include <utility>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -28,6 +30,12 @@ struct Context {
   void *mask_nom = nullptr;
   int *mask_csum = nullptr;
   long mask_cap = 0;
+  // scratch of the per-kernel training entry points: the "next" Ci / Cj of the fused kernel
+  void *trace_next = nullptr;
+  long trace_cap = 0;  // elements of 8 bytes
+  // partial sums of the split-K forward, shared by every caller (stream order serialises its use)
+  void *fwd_part = nullptr;
+  size_t fwd_cap = 0;  // bytes
 };
 static Context g_ctx;
 static std::mutex g_ctx_mutex;
@@ -46,7 +54,8 @@ static long g_prof_launches[K_COUNT];
 const char *kernel_name(int id) {
   static const char *names[K_COUNT] = {"forward", "softmax", "counters", "trace_weights", "update_bias",
                                        "update_bias_regularized", "mask_scores", "mask_swap",
-                                       "mask_fix_weights", "apply_mask", "argmax", "gather_rows", "fill"};
+                                       "mask_fix_weights", "apply_mask", "argmax", "gather_rows", "fill",
+                                       "train_fused"};
   return (id >= 0 && id < K_COUNT) ? names[id] : "?";
 }
 
@@ -101,12 +110,75 @@ static int ensure_mask_scratch(long N) {
   return 0;
 }
 
+static int ensure_trace_scratch(long elems) {
+  if (elems <= g_ctx.trace_cap) return 0;
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  if (g_ctx.trace_next) SB_HIP(hipFree(g_ctx.trace_next));
+  g_ctx.trace_next = nullptr;
+  g_ctx.trace_cap = 0;
+  SB_HIP(hipMalloc(&g_ctx.trace_next, (size_t)elems * sizeof(double)));
+  g_ctx.trace_cap = elems;
+  return 0;
+}
+
+template <typename T>
+static int forward_scratch(long B, long N, long H, long Mc, T **scratch, size_t *elems) {
+  const ForwardPlan plan = forward_plan<T>(B, N, H, Mc);
+  const size_t bytes = (size_t)plan.scratch_elems * sizeof(T);
+  if (bytes > g_ctx.fwd_cap) {
+    SB_HIP(hipStreamSynchronize(g_ctx.stream));
+    if (g_ctx.fwd_part) SB_HIP(hipFree(g_ctx.fwd_part));
+    g_ctx.fwd_part = nullptr;
+    g_ctx.fwd_cap = 0;
+    SB_HIP(hipMalloc(&g_ctx.fwd_part, bytes));
+    g_ctx.fwd_cap = bytes;
+  }
+  *scratch = (T *)g_ctx.fwd_part;
+  *elems = g_ctx.fwd_cap / sizeof(T);
+  return 0;
+}
+
+static bool use_old_train_path() {
+  static const bool v = [] {
+    const char *e = getenv("SB_TRAIN_PATH");
+    return e && std::string(e) == "old";
+  }();
+  return v;
+}
+
+// Per-kernel entry points keep the reference's in-place contract: the fused kernel writes the new
+// Ci / Cj into scratch, which is then copied over the caller's arrays.
+template <typename T>
+static int train_in_place(const T *x, const T *y, T *Cij, T *W, T *Ci, T *Cj, const uint8_t *wmask,
+                          int bias_mode, T *bias, T *kbi, long B, long N, long H, long Mc, T taupdt,
+                          T cthr, T khalf, T pmin, T taubdt) {
+  hipStream_t st = g_ctx.stream;
+  const long M = H * Mc;
+  if (use_old_train_path()) {
+    int rc = launch_counters<T>(st, x, y, Ci, Cj, B, N, M, taupdt, bias_mode, bias, kbi, cthr, khalf,
+                                pmin, taubdt);
+    if (rc) return rc;
+    return launch_trace_weights<T>(st, x, y, Cij, W, Ci, Cj, wmask, B, N, H, Mc, taupdt, cthr);
+  }
+  SB_REQUIRE(N > 0 && M > 0, "sizes must be positive");
+  int rc = ensure_trace_scratch(N + M);
+  if (rc) return rc;
+  T *ci_next = (T *)g_ctx.trace_next, *cj_next = ci_next + N;
+  rc = launch_train_fused<T>(st, x, y, Cij, W, Ci, Cj, ci_next, cj_next, wmask, bias_mode, bias, kbi, B,
+                             N, H, Mc, taupdt, cthr, khalf, pmin, taubdt);
+  if (rc) return rc;
+  SB_HIP(hipMemcpyAsync(Ci, ci_next, (size_t)N * sizeof(T), hipMemcpyDeviceToDevice, st));
+  SB_HIP(hipMemcpyAsync(Cj, cj_next, (size_t)M * sizeof(T), hipMemcpyDeviceToDevice, st));
+  return 0;
+}
+
 // ======================================================================================== network
 struct Layer {
   bool plastic = false;
   long N = 0, H = 0, Mc = 0, M = 0;
   double taupdt = 0, pmin = 0, khalf = 0, taubdt = 0;
   void *W = nullptr, *bias = nullptr, *Ci = nullptr, *Cj = nullptr, *Cij = nullptr, *kbi = nullptr;
+  void *Ci_alt = nullptr, *Cj_alt = nullptr;  // the fused training kernel ping-pongs Ci / Cj
   uint8_t *wmask = nullptr;
   void *act = nullptr;  // [act_rows, M]
   long act_rows = 0;
@@ -146,6 +218,8 @@ static int layer_alloc(Layer &L, T ci0, T cj0, T cij0) {
   SB_HIP(hipMalloc(&L.bias, L.M * sizeof(T)));
   SB_HIP(hipMalloc(&L.Cj, L.M * sizeof(T)));
   SB_HIP(hipMalloc(&L.Ci, L.N * sizeof(T)));
+  SB_HIP(hipMalloc(&L.Cj_alt, L.M * sizeof(T)));
+  SB_HIP(hipMalloc(&L.Ci_alt, L.N * sizeof(T)));
   int rc = 0;
   if ((rc = launch_fill<T>(st, (T *)L.W, T(0), nm))) return rc;
   if ((rc = launch_fill<T>(st, (T *)L.Cij, cij0, nm))) return rc;
@@ -168,7 +242,7 @@ static int layer_free(Layer &L) {
   void *w = L.wmask, *c = L.csum;
   rc |= free_dev(L.W); rc |= free_dev(L.bias); rc |= free_dev(L.Ci); rc |= free_dev(L.Cj);
   rc |= free_dev(L.Cij); rc |= free_dev(L.kbi); rc |= free_dev(w); rc |= free_dev(L.act);
-  rc |= free_dev(L.nom); rc |= free_dev(c);
+  rc |= free_dev(L.nom); rc |= free_dev(c); rc |= free_dev(L.Ci_alt); rc |= free_dev(L.Cj_alt);
   L.wmask = nullptr; L.csum = nullptr;
   return rc;
 }
@@ -187,8 +261,12 @@ static int ensure_act(sb_net *net, long rows) {
 
 template <typename T>
 static int layer_forward(const Layer &L, const T *x, long B) {
+  T *scratch = nullptr;
+  size_t elems = 0;
+  int rc = forward_scratch<T>(B, L.N, L.H, L.Mc, &scratch, &elems);
+  if (rc) return rc;
   return launch_forward<T>(g_ctx.stream, (T *)L.act, x, (const T *)L.W, (const T *)L.bias, B, L.N, L.H,
-                           L.Mc, true);
+                           L.Mc, true, scratch, elems);
 }
 
 // One training step of `L` on input x (and on y = its own activation or the labels), in the order of
@@ -199,11 +277,23 @@ static int layer_train_step(Layer &L, const T *x, const T *y, long B, long h) {
   hipStream_t st = g_ctx.stream;
   const T tau = (T)L.taupdt;
   const T cthr = (T)(L.taupdt / 2);
-  int rc = launch_counters<T>(st, x, y, (T *)L.Ci, (T *)L.Cj, B, L.N, L.M, tau, L.plastic ? 1 : 0,
-                              (T *)L.bias, (T *)L.kbi, cthr, (T)L.khalf, (T)L.pmin, (T)L.taubdt);
-  if (rc) return rc;
-  rc = launch_trace_weights<T>(st, x, y, (T *)L.Cij, (T *)L.W, (const T *)L.Ci, (const T *)L.Cj,
-                               L.plastic ? L.wmask : nullptr, B, L.N, L.H, L.Mc, tau, cthr);
+  int rc = 0;
+  if (use_old_train_path()) {
+    rc = launch_counters<T>(st, x, y, (T *)L.Ci, (T *)L.Cj, B, L.N, L.M, tau, L.plastic ? 1 : 0,
+                            (T *)L.bias, (T *)L.kbi, cthr, (T)L.khalf, (T)L.pmin, (T)L.taubdt);
+    if (rc) return rc;
+    rc = launch_trace_weights<T>(st, x, y, (T *)L.Cij, (T *)L.W, (const T *)L.Ci, (const T *)L.Cj,
+                                 L.plastic ? L.wmask : nullptr, B, L.N, L.H, L.Mc, tau, cthr);
+  } else {
+    rc = launch_train_fused<T>(st, x, y, (T *)L.Cij, (T *)L.W, (const T *)L.Ci, (const T *)L.Cj,
+                               (T *)L.Ci_alt, (T *)L.Cj_alt, L.plastic ? L.wmask : nullptr,
+                               L.plastic ? 1 : 0, (T *)L.bias, (T *)L.kbi, B, L.N, L.H, L.Mc, tau, cthr,
+                               (T)L.khalf, (T)L.pmin, (T)L.taubdt);
+    if (!rc) {
+      std::swap(L.Ci, L.Ci_alt);
+      std::swap(L.Cj, L.Cj_alt);
+    }
+  }
   if (rc) return rc;
   if (L.plastic && h >= 0) {
     rc = launch_update_mask<T>(st, L.wmask, (const T *)nullptr, (const T *)L.Ci, (const T *)L.Cj,
@@ -422,6 +512,8 @@ int sb_shutdown(void) {
   SB_HIP(hipStreamSynchronize(g_ctx.stream));
   if (g_ctx.mask_nom) SB_HIP(hipFree(g_ctx.mask_nom));
   if (g_ctx.mask_csum) SB_HIP(hipFree(g_ctx.mask_csum));
+  if (g_ctx.trace_next) SB_HIP(hipFree(g_ctx.trace_next));
+  if (g_ctx.fwd_part) SB_HIP(hipFree(g_ctx.fwd_part));
   SB_HIP(hipStreamDestroy(g_ctx.stream));
   g_ctx = Context();
   return 0;
@@ -480,7 +572,7 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
 #define SB_DEFINE_KERNEL_API(SFX, T)                                                                   \
   int sb_update_state_##SFX(T *act, const T *x, const T *W, const T *bias, long B, long N, long M) {   \
     SB_READY();                                                                                        \
-    return launch_forward<T>(g_ctx.stream, act, x, W, bias, B, N, 1, M, false);                        \
+    return launch_forward<T>(g_ctx.stream, act, x, W, bias, B, N, 1, M, false, (T *)nullptr, 0);       \
   }                                                                                                    \
   int sb_softmax_minicolumns_##SFX(T *act, long B, long H, long Mc) {                                  \
     SB_READY();                                                                                        \
@@ -489,16 +581,18 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
   int sb_compute_activation_##SFX(T *act, const T *x, const T *W, const T *bias, long B, long N,       \
                                   long H, long Mc) {                                                   \
     SB_READY();                                                                                        \
-    return launch_forward<T>(g_ctx.stream, act, x, W, bias, B, N, H, Mc, true);                        \
+    SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");                           \
+    T *scratch = nullptr;                                                                              \
+    size_t elems = 0;                                                                                  \
+    int rc = forward_scratch<T>(B, N, H, Mc, &scratch, &elems);                                        \
+    if (rc) return rc;                                                                                 \
+    return launch_forward<T>(g_ctx.stream, act, x, W, bias, B, N, H, Mc, true, scratch, elems);        \
   }                                                                                                    \
   int sb_update_weights_##SFX(T *Ci, T *Cj, T *Cij, const T *a_i, const T *a_o, T taupdt, T *W,        \
                               T cthr, long B, long N, long M) {                                        \
     SB_READY();                                                                                        \
-    int rc = launch_counters<T>(g_ctx.stream, a_i, a_o, Ci, Cj, B, N, M, taupdt, 0, nullptr, nullptr,  \
-                                cthr, T(0), T(0), T(0));                                               \
-    if (rc) return rc;                                                                                 \
-    return launch_trace_weights<T>(g_ctx.stream, a_i, a_o, Cij, W, Ci, Cj, nullptr, B, N, 1, M,        \
-                                   taupdt, cthr);                                                      \
+    return train_in_place<T>(a_i, a_o, Cij, W, Ci, Cj, nullptr, 0, nullptr, nullptr, B, N, 1, M, taupdt, \
+                             cthr, T(0), T(0), T(0));                                                  \
   }                                                                                                    \
   int sb_update_bias_##SFX(T *bias, const T *Cj, T cthr, long M) {                                     \
     SB_READY();                                                                                        \
@@ -537,11 +631,8 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
     SB_REQUIRE(N > 0 && H > 0 && Mc > 0, "sizes must be positive");                                    \
     SB_REQUIRE(h < H, "hypercolumn index out of range");                                               \
     const T cthr = (T)((double)taupdt / 2);                                                            \
-    int rc = launch_counters<T>(g_ctx.stream, x, y, Ci, Cj, B, N, H * Mc, taupdt, 1, bias, kbi, cthr,  \
-                                khalf, pmin, taubdt);                                                  \
-    if (rc) return rc;                                                                                 \
-    rc = launch_trace_weights<T>(g_ctx.stream, x, y, Cij, W, Ci, Cj, wmask, B, N, H, Mc, taupdt,       \
-                                 cthr);                                                                \
+    int rc = train_in_place<T>(x, y, Cij, W, Ci, Cj, wmask, 1, bias, kbi, B, N, H, Mc, taupdt, cthr,     \
+                               khalf, pmin, taubdt);                                                   \
     if (rc || h < 0) return rc;                                                                        \
     if ((rc = ensure_mask_scratch(N))) return rc;                                                      \
     rc = launch_update_mask<T>(g_ctx.stream, wmask, (const T *)nullptr, Ci, Cj, Cij, cthr, N, H, Mc,   \

@@ -148,7 +148,7 @@ def _mask_problem(rng, N, H, Mc, dtype, density=0.1):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("N,H,Mc", [(1, 1, 2), (7, 2, 3), (128, 5, 20), (1568, 30, 100), (5000, 3, 4)])
+@pytest.mark.parametrize("N,H,Mc", [(1, 1, 2), (7, 2, 3), (128, 5, 20), (1568, 30, 100), (5000, 3, 4), (9000, 2, 3)])
 @pytest.mark.parametrize("iterations", [0, 1, 16])
 def test_update_mask_bit_exact(k, oracle, dtype, N, H, Mc, iterations):
     rng = np.random.default_rng(N + H + Mc)
