@@ -117,21 +117,40 @@ class GpuRun:
     def sync(self):
         self.capi.check(self.lib.sb_sync())
 
+    def classifier_steps(self, n_steps):
+        """Training steps of the 10-class dense layer (forward of the hidden layer + its fused trace and
+        weight update on the labels), batches [0, n_steps) of one epoch; returns the number of samples."""
+        n_steps = min(n_steps, self.nb)
+        perm = self.rng.permutation(self.ns).astype(np.int64)
+        self.capi.check(self.lib.sb_net_train_batches(self.net, 1, BATCH, perm.ctypes.data, None, 0, 0,
+                                                      n_steps, 1))
+        return sum(min(BATCH, self.ns - b * BATCH) for b in range(n_steps))
+
+    def evaluate(self, x, y):
+        correct, total = ctypes.c_int64(0), ctypes.c_int64(0)
+        self.capi.check(self.lib.sb_net_evaluate(self.net, x.ctypes.data, y.ctypes.data, x.shape[0],
+                                                 x.shape[1], y.shape[1], BATCH, ctypes.byref(correct),
+                                                 ctypes.byref(total), None))
+        return correct.value, total.value
+
     def profile(self, first_step, n_steps):
         self.capi.check(self.lib.sb_profile_start())
         self.run_steps(first_step, n_steps)
         self.capi.check(self.lib.sb_profile_stop())
         out = {}
+        self.raw_bracket_ms, self.brackets = 0.0, 0
         for k in range(self.lib.sb_profile_kernels()):
             ms, n = ctypes.c_double(0), ctypes.c_long(0)
             self.capi.check(self.lib.sb_profile_get(k, ctypes.byref(ms), ctypes.byref(n)))
+            self.raw_bracket_ms += ms.value
+            self.brackets += n.value
             if n.value:
                 out[self.lib.sb_profile_kernel_name(k).decode()] = {
                     "launches": n.value, "avg_us": 1e3 * ms.value / n.value}
         return out
 
 
-def cpu_baseline(x, y, budget_s=20.0, max_steps=40):
+def cpu_baseline(x, y, budget_s=15.0, max_steps=100000):
     """The CPU oracle (reference loop structure, reference flag set, OpenMP) on the first steps of the
     same workload: same initial state, same data, batches in storage order, rewiring every 15th step."""
     from oracle.oracle import Oracle
@@ -140,7 +159,10 @@ def cpu_baseline(x, y, budget_s=20.0, max_steps=40):
     tau, cthr = HP["l1_taupdt"], HP["l1_taupdt"] / 2
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
 
+    full_batches = x.shape[0] // BATCH
+
     def step(i):
+        i = i % full_batches
         xb = x[i * BATCH:(i + 1) * BATCH]
         act = np.zeros((xb.shape[0], H * MC), dtype=np.float32)
         o.update_state(act, st["weights"], st["bias"], xb)
@@ -166,6 +188,35 @@ def cpu_baseline(x, y, budget_s=20.0, max_steps=40):
             "ms_per_step": 1e3 * dt / max(steps, 1)}
 
 
+def measured_traffic():
+    """HBM bytes per launch of the dominant kernel, as measured with rocprofv3 --pmc FETCH_SIZE /
+    WRITE_SIZE and recorded in profiles/ (line `traffic_bytes_per_launch: N`); None when absent."""
+    path = os.path.join(ROOT, "profiles", "k_train_fused_mnist_f32_b128_pmc.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return float(line.split(":", 1)[1])
+    except OSError:
+        pass
+    return None
+
+
+def copy_calibration(nbytes=64 << 20, copies=6):
+    from streambrain_amd import _capi
+    from streambrain_amd._capi import DeviceArray
+    _capi.init(0)
+    lib = _capi.lib()
+    src, dst = DeviceArray((nbytes,), np.uint8), DeviceArray((nbytes,), np.uint8)
+    _capi.check(lib.sb_fill_bytes(src.ptr, 1, nbytes))
+    _capi.check(lib.sb_fill_bytes(dst.ptr, 2, nbytes))
+    for _ in range(copies):
+        _capi.check(lib.sb_memcpy_d2d(dst.ptr, src.ptr, nbytes))
+    _capi.check(lib.sb_sync())
+    print(json.dumps({"copy_calibration": {"copies": copies, "bytes_read_per_copy": nbytes,
+                                           "bytes_written_per_copy": nbytes}}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -173,11 +224,17 @@ def main():
     ap.add_argument("--warmup", type=int, default=60)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--samples", type=int, default=N_SAMPLES)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run six 64 MiB device-to-device copies: the known-size kernel that "
+                         "hardware counter readings (FETCH_SIZE, WRITE_SIZE) are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
               "(the path is not sharded across devices)", file=sys.stderr)
         return 2
+
+    if args.copy_calibration:
+        return copy_calibration()
 
     x, y = synthetic_dataset(args.samples)
     run = GpuRun(x, y)
@@ -189,7 +246,28 @@ def main():
     run.sync()
     dt = time.perf_counter() - t0
 
-    prof = run.profile(args.warmup + args.steps, min(args.steps, 2 * run.nb))
+    # Per-kernel durations: every launch of a second pass over the same number of steps is bracketed by
+    # HIP events on the library's stream.  A bracket adds a little to each launch; how much is calibrated
+    # from the two passes themselves: (sum of all brackets - wall time of the unbracketed pass) / brackets.
+    n_prof = min(args.steps, 2 * run.nb)
+    prof = run.profile(args.warmup + args.steps, n_prof)
+    bracket_us = max(0.0, (1e3 * run.raw_bracket_ms - 1e6 * dt * n_prof / args.steps) / max(run.brackets, 1))
+    for k in prof.values():
+        k["raw_avg_us"] = k["avg_us"]
+        k["avg_us"] = max(k["avg_us"] - bracket_us, 0.0)
+
+    # the two other phases of the reference's example run, reported beside the headline figure
+    run.classifier_steps(20)
+    run.sync()
+    t1 = time.perf_counter()
+    cls_samples = run.classifier_steps(run.nb)
+    run.sync()
+    cls_dt = time.perf_counter() - t1
+    xt, yt = x[:10000], y[:10000]
+    run.evaluate(xt[:BATCH], yt[:BATCH])
+    t2 = time.perf_counter()
+    run.evaluate(xt, yt)
+    ev_dt = time.perf_counter() - t2
     n, m = 2 * N_PIXELS, H * MC
     tw = prof.get("train_fused") or prof.get("trace_weights") or {"avg_us": float("nan")}
     alg_bytes = 3 * 4 * n * m  # read Cij, write Cij, write W: 12 bytes per synapse
@@ -215,12 +293,18 @@ def main():
                    "batch": BATCH, "in_features": n, "hypercolumns": H, "minicolumns": MC,
                    "samples": args.samples},
         "roofline": {"bound": "hbm", "kernel": "k_train_fused", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(),
                      "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": tw["avg_us"]},
         "mfma": {"kernel": "k_forward", "achieved_tflops": fwd_tflops, "peak_tflops": 157.3,
                  "frac": fwd_tflops / 157.3, "avg_launch_us": fwd["avg_us"],
                  "trace_gemm_tflops_in_fused_kernel": 2.0 * BATCH * n * m / (tw["avg_us"] * 1e-6) / 1e12},
         "kernels": prof,
+        "event_bracket_overhead_us": {"calibrated": bracket_us,
+                                      "empty_bracket": run.lib.sb_profile_bracket_overhead_us()},
+        "other_phases": {
+            "classifier_layer_train_samples_per_s": cls_samples / cls_dt,
+            "evaluate_samples_per_s_host_images_pcie_inclusive": xt.shape[0] / ev_dt,
+        },
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(x, y)

@@ -208,10 +208,15 @@ int sb_net_forward(sb_net *net, const void *h_images, long n_rows, long n_featur
  * Between sb_profile_start and sb_profile_stop every kernel launch of the library is bracketed by HIP
  * events on the library's stream; afterwards sb_profile_get returns, per kernel index in
  * [0, sb_profile_kernels()), the summed elapsed time and the number of launches.  The reference has no
- * counterpart (it times whole runs with time.time(), train.py:181-193). */
+ * counterpart (it times whole runs with time.time(), train.py:181-193).  The sums are raw bracket times:
+ * a bracket adds a few microseconds of its own to a short kernel (compare the bracketed sum of a run
+ * with its unbracketed wall time to calibrate). */
 int sb_profile_start(void);
 int sb_profile_stop(void);
 int sb_profile_kernels(void);
+/* Elapsed time of an empty event bracket as measured by the last sb_profile_start: an upper bound of
+ * what a bracket adds to a launch. */
+double sb_profile_bracket_overhead_us(void);
 const char *sb_profile_kernel_name(int kernel);
 int sb_profile_get(int kernel, double *total_ms, long *launches);
 

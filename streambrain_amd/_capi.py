@@ -62,7 +62,8 @@ _PLAIN_SIGS = {
     "sb_net_forward": [_P, _P, _L, _L, _I, _L, _P],
 }
 _RESTYPES = {"sb_last_error": ctypes.c_char_p, "sb_stream": _P}
-_OTHER_SIGS = {"sb_profile_kernel_name": ([_I], ctypes.c_char_p)}
+_OTHER_SIGS = {"sb_profile_kernel_name": ([_I], ctypes.c_char_p),
+               "sb_profile_bracket_overhead_us": ([], _D)}
 
 
 def exported_symbols():

@@ -2,6 +2,7 @@
 // device-resident network object.  Host code only; kernels live in sb_kernels.hpp.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <utility>
@@ -50,6 +51,7 @@ static std::vector<ProfRecord> g_prof_records;
 static std::vector<hipEvent_t> g_prof_pool;
 static double g_prof_ms[K_COUNT];
 static long g_prof_launches[K_COUNT];
+static double g_prof_overhead_ms = 0;  // elapsed time of an empty event bracket
 
 const char *kernel_name(int id) {
   static const char *names[K_COUNT] = {"forward", "softmax", "counters", "trace_weights", "update_bias",
@@ -807,6 +809,29 @@ int sb_profile_start(void) {
     g_prof_ms[k] = 0;
     g_prof_launches[k] = 0;
   }
+  // what a bracket costs at most: median elapsed time of event pairs with nothing in between (reported
+  // by sb_profile_bracket_overhead_us; the per-kernel sums stay raw)
+  {
+    constexpr int kPairs = 33;
+    hipEvent_t ev[2 * kPairs];
+    for (auto &e : ev) e = prof_event();
+    for (int i = 0; i < kPairs; i++) {
+      if (!ev[2 * i] || !ev[2 * i + 1]) continue;
+      SB_HIP(hipEventRecord(ev[2 * i], g_ctx.stream));
+      SB_HIP(hipEventRecord(ev[2 * i + 1], g_ctx.stream));
+    }
+    SB_HIP(hipStreamSynchronize(g_ctx.stream));
+    std::vector<float> gaps;
+    for (int i = 0; i < kPairs; i++) {
+      float ms = 0;
+      if (ev[2 * i] && ev[2 * i + 1] && hipEventElapsedTime(&ms, ev[2 * i], ev[2 * i + 1]) == hipSuccess)
+        gaps.push_back(ms);
+    }
+    for (auto &e : ev)
+      if (e) g_prof_pool.push_back(e);
+    std::sort(gaps.begin(), gaps.end());
+    g_prof_overhead_ms = gaps.empty() ? 0.0 : gaps[gaps.size() / 2];
+  }
   g_prof_on = true;
   return 0;
 }
@@ -828,6 +853,8 @@ int sb_profile_stop(void) {
 }
 
 int sb_profile_kernels(void) { return K_COUNT; }
+
+double sb_profile_bracket_overhead_us(void) { return 1e3 * g_prof_overhead_ms; }
 
 const char *sb_profile_kernel_name(int kernel) { return kernel_name(kernel); }
 
