@@ -2,8 +2,8 @@
 BCPNN_BACKEND environment variable picks the module whose DenseLayer, StructuralPlasticityLayer and
 Network become the package's API, so a StreamBrain training script runs unchanged.
 
-This repository ships one backend, `hip` (MI355X); it is also the default.  The one-line addition a
-StreamBrain checkout needs to select it is shown in INTEGRATION.md.
+This repository ships one backend, `hip` (MI355X); it is also the default.  A StreamBrain checkout
+selects it by adding the same `elif _BACKEND == 'hip'` branch to its own dispatcher.
 """
 import os
 import sys

@@ -3,7 +3,7 @@
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 
-Workload (BASELINE.json configs[1]): MNIST-shaped 2-layer network, float32, batch 128, 60000 seeded
+Workload: the MNIST-shaped 2-layer network, float32, batch 128, 60000 seeded
 synthetic samples; input 784 pixels complementary-coded to 1568 units (~19% nonzero pixels, uniform
 in (0,1]); hidden layer 30 hypercolumns x 100 minicolumns with a receptive-field mask of density 0.1;
 10-class dense output layer.  A "step" is one structural-plasticity-layer training step on one
