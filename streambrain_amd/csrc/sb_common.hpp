@@ -29,10 +29,13 @@ struct Real<float> {
   }
   static __device__ __forceinline__ int acc_row(int q, int v) { return 4 * q + v; }
   static __device__ __forceinline__ float log_(float x) { return logf(x); }
-  // log for the weight recompute: the hardware log2 (1 ulp, v_log_f32) scaled by ln 2; arguments
-  // below the normal range, where that instruction flushes, take the library routine
+  // log for the weight recompute: the hardware log2 (1 ulp, v_log_f32) scaled by ln 2.  That
+  // instruction flushes arguments below the normal range, so small arguments are scaled by 2^32 first
+  // and 32 ln 2 is taken off again.
   static __device__ __forceinline__ float wlog(float x) {
-    return x >= 1.17549435e-38f ? __builtin_amdgcn_logf(x) * 0.693147180559945309f : logf(x);
+    const bool tiny = x < 0x1p-96f;
+    const float l2 = __builtin_amdgcn_logf(x * (tiny ? 0x1p32f : 1.0f));
+    return __builtin_fmaf(l2, 0.693147180559945309f, tiny ? -32.0f * 0.693147180559945309f : 0.0f);
   }
   static __device__ __forceinline__ float exp_(float x) { return expf(x); }
   // single IEEE operations: the pragma keeps the compiler from contracting them into FMAs
@@ -122,6 +125,36 @@ __device__ __forceinline__ void load_vw_sel(T (&out)[Real<T>::VW], const T *p, c
   for (int e = 0; e < VW; e++) out[e] = ok ? v[e] : T(0);
 }
 
+// Branch-free loads in two halves, for code that wants many loads in flight before the first use.
+// load_vw_raw issues the loads of base[off + col .. off + col + VW) -- from element 0 of the array where
+// the guard fails, so `base` must point to at least one valid (for VEC: 16-byte aligned) vector -- and
+// zero_invalid, called where the values are consumed, zeroes what the guard excludes.  (A select right
+// behind the load would make the compiler wait for the load there.)
+template <typename T, bool VEC>
+__device__ __forceinline__ void load_vw_raw(T (&out)[Real<T>::VW], const T *base, long off, long col,
+                                            long limit, bool row_ok) {
+  constexpr int VW = Real<T>::VW;
+  if (VEC) {
+    const bool ok = row_ok && col < limit;
+    const typename Real<T>::vec_t v =
+        *reinterpret_cast<const typename Real<T>::vec_t *>(base + (ok ? off + col : 0));
+#pragma unroll
+    for (int e = 0; e < VW; e++) out[e] = v[e];
+  } else {
+#pragma unroll
+    for (int e = 0; e < VW; e++) out[e] = base[(row_ok && col + e < limit) ? off + col + e : 0];
+  }
+}
+template <typename T, bool VEC>
+__device__ __forceinline__ void zero_invalid(T (&v)[Real<T>::VW], long col, long limit, bool row_ok) {
+  constexpr int VW = Real<T>::VW;
+#pragma unroll
+  for (int e = 0; e < VW; e++) {
+    const bool ok = VEC ? (row_ok && col < limit) : (row_ok && col + e < limit);
+    v[e] = ok ? v[e] : T(0);
+  }
+}
+
 // Width-generic variants: W consecutive elements (W = 1, 2, 4 for float; 1, 2 for double), moved as one
 // W*sizeof(T)-byte access when VEC promises that alignment and limit % W == 0.
 template <typename T, int W>
@@ -167,7 +200,7 @@ __device__ __forceinline__ T trace_reciprocal(T c, T cthr) {
 }
 template <typename T>
 __device__ __forceinline__ T weight_from_traces(T cij, T rci, T rcj, T cthr4) {
-  const T num = cij > cthr4 ? cij : cthr4;
+  const T num = fmax(cij, cthr4);  // cthr4 as well when cij is NaN, like `cij > cthr4 ? cij : cthr4`
   const T w = Real<T>::wlog(num * rci * rcj);
   return (rci < T(0) || rcj < T(0)) ? T(0) : w;
 }

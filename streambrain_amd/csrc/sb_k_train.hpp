@@ -25,7 +25,14 @@
 //   4. The accumulators go through LDS into a row-major layout; each thread then finishes 4 consecutive
 //      columns of 4 rows: decay + clamp, weight, mask, one 16-byte store each to Cij and W.
 #pragma once
+#include <type_traits>
+
 #include "sb_kernels.hpp"
+
+// Hook for phase timing in development builds; expands to nothing in the library.
+#ifndef SB_PHASE_MARK
+#define SB_PHASE_MARK(n)
+#endif
 
 namespace sb {
 
@@ -48,7 +55,9 @@ struct TrainArgs {
   long tiles_i, tiles_j;
 };
 
-template <typename T, int KCH, bool VEC>
+// MB: mask bytes fetched per vector of VW columns -- 1 when Mc is a multiple of VW (every vector lies
+// inside one hypercolumn), VW otherwise.
+template <typename T, int KCH, bool VEC, int MB>
 __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   using R = Real<T>;
   using acc_t = typename R::acc_t;
@@ -60,11 +69,14 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   constexpr int SP = KCH / RPP;         // staging passes per chunk
   constexpr int CP = TS + VW;           // pitch of the accumulator tile in LDS
   static_assert(KCH % RPP == 0 && KCH % 4 == 0, "chunk size");
-  constexpr int SLAB = 2 * KCH * TS > TS * CP ? 2 * KCH * TS : TS * CP;  // staging, then accumulators
+  // LDS: the staging slabs xs | ys; once they are consumed the same memory holds the accumulator tile
+  // followed by the trace reciprocals of the tile's rows and columns
+  constexpr int TAIL = TS * CP + 2 * TS;
+  constexpr int SLAB = 2 * KCH * TS > TAIL ? 2 * KCH * TS : TAIL;
 
-  __shared__ __attribute__((aligned(16))) T slab[SLAB];  // xs | ys, later the accumulator tile
-  __shared__ T rci_s[TS], rcj_s[TS];
+  __shared__ __attribute__((aligned(16))) T slab[SLAB];
   T *xs = slab, *ys = slab + KCH * TS;
+  T *rci_s = slab + TS * CP, *rcj_s = rci_s + TS;
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, p = lane & 15, q = lane >> 4;
   const long it = (long)blockIdx.x / a.tiles_j, jt = (long)blockIdx.x % a.tiles_j;
@@ -74,44 +86,21 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   const int eg = tid % G, er = tid / G;
   const long ecol = j0 + VW * eg;
 
-  // ---- 1. Cij prefetch
-  T cpre[PASSES][VW];
+  SB_PHASE_MARK(0);
+  // All global loads are branch-free (clamped addresses; what a guard excludes is zeroed or ignored
+  // where it is consumed), so they stay in flight together.  Loads return in issue order, hence the
+  // order below: first what the first MFMA needs (chunk 0 of x and y, mostly L2 hits), and the Cij
+  // tile (HBM) only while the second-to-last chunk is being computed.
+  T sx[SP][VW], sy[SP][VW];
+  auto request_chunk = [&](long b0) {
 #pragma unroll
-  for (int k = 0; k < PASSES; k++) {
-    const long row = i0 + er + RPP * k;
-    load_vw<T, VEC>(cpre[k], a.Cij + row * a.M, ecol, a.M, row < a.N);
-  }
-
-  // mask bits of the thread's PASSES x VW synapses, requested now for the same reason
-  uint32_t onbits = 0xffffffffu;
-  if (a.wmask) {
-    uint32_t hc[VW];
-#pragma unroll
-    for (int e = 0; e < VW; e++) hc[e] = (ecol + e < a.M) ? (uint32_t)(ecol + e) / (uint32_t)a.Mc : 0u;
-    // the VW columns usually sit in one hypercolumn: then one mask byte serves the vector
-    const bool one_hc = (ecol + VW - 1 < a.M) && hc[0] == hc[VW - 1];
-    onbits = 0;
-#pragma unroll
-    for (int k = 0; k < PASSES; k++) {
-      const long row = i0 + er + RPP * k;
-      if (row >= a.N) continue;
-      const uint8_t *mrow = a.wmask + row * a.H;
-      if (one_hc) {
-        if (mrow[hc[0]] != 0) onbits |= ((1u << VW) - 1u) << (VW * k);
-      } else {
-#pragma unroll
-        for (int e = 0; e < VW; e++)
-          if (ecol + e < a.M && mrow[hc[e]] != 0) onbits |= 1u << (VW * k + e);
-      }
+    for (int m = 0; m < SP; m++) {
+      const long b = b0 + er + RPP * m;
+      load_vw_raw<T, VEC>(sx[m], a.x, b * a.N, i0 + VW * eg, a.N, b < a.B);
+      load_vw_raw<T, VEC>(sy[m], a.y, b * a.M, ecol, a.M, b < a.B);
     }
-  }
-
-  acc_t acc[2][2];
-#pragma unroll
-  for (int r = 0; r < 2; r++)
-#pragma unroll
-    for (int c = 0; c < 2; c++) acc[r][c] = acc_t{0, 0, 0, 0};
-  const int iw = (w >> 1) * 32, jw = (w & 1) * 32;  // sub-tile of this wavefront
+  };
+  request_chunk(0);
 
   // column sums: lanes 0..31 of wavefronts 0,1 take the 64 x columns, of wavefronts 2,3 the y columns
   const bool summer = lane < 32;
@@ -121,23 +110,53 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   const long sidx = (sum_i ? i0 : j0) + scol;
   const bool sum_ok = summer && sidx < (sum_i ? a.N : a.M);
   const bool writes_bias = sum_ok && !sum_i && it == 0 && a.bias_mode == 1;
-  const T cold = sum_ok ? (sum_i ? a.Ci : a.Cj)[sidx] : T(1);  // old trace, requested early
-  T kb = writes_bias ? a.kbi[sidx] : T(1);
+  const T cold = (sum_i ? a.Ci : a.Cj)[sum_ok ? sidx : 0];  // old trace
+  T kb = T(1);
+  if (a.bias_mode == 1) kb = a.kbi[writes_bias ? sidx : 0];
   T csum = T(0);
 
-  // ---- 2./3. chunks of the batch
-  for (long b0 = 0; b0 < a.B; b0 += KCH) {
-    const long rows = a.B - b0 < KCH ? a.B - b0 : KCH;
-    if (b0 > 0) __syncthreads();  // previous chunk fully consumed
-    T sx[SP][VW], sy[SP][VW];
+  // mask bytes of the thread's PASSES x VW synapses: a small, L2-resident array, fetched up front
+  uint32_t mb[PASSES][MB];
+  if (a.wmask) {
+    uint32_t hc[MB];
 #pragma unroll
-    for (int m = 0; m < SP; m++) {
-      const long b = b0 + er + RPP * m;
-      load_vw<T, VEC>(sx[m], a.x + b * a.N, i0 + VW * eg, a.N, b < a.B);
-      load_vw<T, VEC>(sy[m], a.y + b * a.M, ecol, a.M, b < a.B);
+    for (int e = 0; e < MB; e++) hc[e] = ecol + e < a.M ? (uint32_t)(ecol + e) / (uint32_t)a.Mc : 0u;
+#pragma unroll
+    for (int k = 0; k < PASSES; k++) {
+      const long row = i0 + er + RPP * k;
+#pragma unroll
+      for (int e = 0; e < MB; e++) mb[k][e] = a.wmask[row < a.N ? row * a.H + hc[e] : 0];
+    }
+  }
+
+  T cpre[PASSES][VW];  // Cij tile: VW columns of PASSES rows per thread
+  auto request_tile = [&]() {
+#pragma unroll
+    for (int k = 0; k < PASSES; k++) {
+      const long row = i0 + er + RPP * k;
+      load_vw_raw<T, VEC>(cpre[k], a.Cij, row * a.M, ecol, a.M, row < a.N);  // excluded parts are never stored
+    }
+  };
+
+  acc_t acc[2][2];
+#pragma unroll
+  for (int r = 0; r < 2; r++)
+#pragma unroll
+    for (int c = 0; c < 2; c++) acc[r][c] = acc_t{0, 0, 0, 0};
+  const int iw = (w >> 1) * 32, jw = (w & 1) * 32;  // sub-tile of this wavefront
+
+  // ---- chunks of the batch.  The loads of chunk c+1 are issued before chunk c is consumed from LDS,
+  // so their latency hides behind the MFMA loop and the column sums.
+  auto chunk = [&](long b0, auto with_tile) {
+    if (b0 > 0) {
+      __syncthreads();  // previous chunk fully consumed
+      SB_PHASE_MARK(2 * (int)(b0 / KCH));
     }
 #pragma unroll
     for (int m = 0; m < SP; m++) {
+      const long b = b0 + er + RPP * m;
+      zero_invalid<T, VEC>(sx[m], i0 + VW * eg, a.N, b < a.B);
+      zero_invalid<T, VEC>(sy[m], ecol, a.M, b < a.B);
       typename R::vec_t vx, vy;
 #pragma unroll
       for (int e = 0; e < VW; e++) {
@@ -148,17 +167,19 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
       *reinterpret_cast<typename R::vec_t *>(&ys[(er + RPP * m) * TS + VW * eg]) = vy;
     }
     __syncthreads();
+    SB_PHASE_MARK(1 + 2 * (int)(b0 / KCH));
+    request_chunk(b0 + KCH);  // past the batch: clamped loads nobody consumes
+    if (decltype(with_tile)::value) request_tile();
 
     if (summer) {
       // rows past the end of the batch were staged as zeros: adding them changes nothing, so the loop
-      // needs no guard; 32 LDS reads are in flight before the (ordered) additions consume them
-      (void)rows;
-      for (int r = 0; r < KCH; r += 32) {
-        T v[32];
+      // needs no guard; 16 LDS reads are in flight before the (ordered) additions consume them
+      for (int r = 0; r < KCH; r += 16) {
+        T v[16];
 #pragma unroll
-        for (int k = 0; k < 32; k++) v[k] = sbase[(r + k) * TS];
+        for (int k = 0; k < 16; k++) v[k] = sbase[(r + k) * TS];
 #pragma unroll
-        for (int k = 0; k < 32; k++) csum = R::add(csum, v[k]);
+        for (int k = 0; k < 16; k++) csum = R::add(csum, v[k]);
       }
     }
 
@@ -174,7 +195,15 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
       acc[1][0] = R::mfma(x1, y0, acc[1][0]);
       acc[1][1] = R::mfma(x1, y1, acc[1][1]);
     }
-  }
+  };
+  long b0 = 0;
+  for (; b0 + 2 * KCH < a.B; b0 += KCH) chunk(b0, std::false_type{});
+  chunk(b0, std::true_type{});  // second-to-last (or only) chunk: the Cij tile is requested here
+  b0 += KCH;
+  if (b0 < a.B) chunk(b0, std::false_type{});
+
+  __syncthreads();  // slabs consumed: their memory is reused from here on
+  SB_PHASE_MARK(12);
 
   // ---- 3. new traces of this tile's rows and columns (reference order of operations)
   if (summer) {
@@ -196,7 +225,6 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
     }
     (sum_i ? rci_s : rcj_s)[scol] = trace_reciprocal<T>(cnew, a.cthr);
   }
-  __syncthreads();  // slabs consumed, reciprocals published
 
   // ---- 4. accumulators -> row-major LDS tile
   T *cs = slab;
@@ -208,9 +236,12 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
       cs[row * CP + jw + 2 * p] = acc[r][0][v];
       cs[row * CP + jw + 2 * p + 1] = acc[r][1][v];
     }
-  __syncthreads();
+  __syncthreads();  // accumulator tile and reciprocals published
+  SB_PHASE_MARK(13);
 
   // ---- epilogue: decay + clamp, weight, mask, stores
+  const T scale = a.invB * a.tau;
+  const bool masked = a.wmask != nullptr;
   T rcj[VW];
 #pragma unroll
   for (int e = 0; e < VW; e++) rcj[e] = rcj_s[VW * eg + e];
@@ -223,17 +254,17 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
     T cv[VW], wv[VW];
 #pragma unroll
     for (int e = 0; e < VW; e++) {
-      T t = cs[lr * CP + VW * eg + e] * a.invB;
-      t = t * a.tau;
-      T cn = cpre[k][e] * a.omt + t;
-      cn = cn > T(0) ? cn : T(0);
+      T cn = cpre[k][e] * a.omt + cs[lr * CP + VW * eg + e] * scale;
+      cn = fmax(cn, T(0));  // 0 as well when cn is NaN, like the reference's `cn > 0 ? cn : 0`
       cv[e] = cn;
       const T wgt = weight_from_traces<T>(cn, rci, rcj[e], a.cthr4);
-      wv[e] = ((onbits >> (VW * k + e)) & 1u) ? wgt : T(0);
+      const bool on = !masked || mb[k][MB == 1 ? 0 : e] != 0;
+      wv[e] = on ? wgt : T(0);
     }
     store_vw<T, VEC>(cv, a.Cij + row * a.M, ecol, a.M);
     store_vw<T, VEC>(wv, a.W + row * a.M, ecol, a.M);
   }
+  SB_PHASE_MARK(14);
 }
 
 }  // namespace sb

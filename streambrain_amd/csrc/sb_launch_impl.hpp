@@ -241,6 +241,9 @@ int launch_trace_weights(hipStream_t st, const T *x, const T *y, T *Cij, T *W, c
 }
 
 // ------------------------------------------------------------------------------------- fused training
+#ifndef SB_TRAIN_KCH
+#define SB_TRAIN_KCH 32
+#endif
 template <typename T>
 int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci, const T *Cj,
                        T *Ci_next, T *Cj_next, const uint8_t *wmask, int bias_mode, T *bias, T *kbi,
@@ -264,13 +267,19 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   const bool vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(y) && aligned16(Cij) &&
                    aligned16(W);
   const dim3 grid((unsigned)(a.tiles_i * a.tiles_j));
-  // batch rows staged per chunk: 32 KiB of LDS per workgroup, so four workgroups share a CU
-  constexpr int KCH = sizeof(T) == 4 ? 64 : 32;
+  SB_REQUIRE(M < (1L << 31), "more than 2^31 output units");
+  // batch rows staged per chunk
+  constexpr int KCH = SB_TRAIN_KCH;
+  const bool one_byte = Mc % VW == 0;  // every vector of VW columns lies inside one hypercolumn
   ProfScope prof_(st, K_TRAIN_FUSED);
-  if (vec)
-    hipLaunchKernelGGL((k_train_fused<T, KCH, true>), grid, dim3(256), 0, st, a);
+  if (vec && one_byte)
+    hipLaunchKernelGGL((k_train_fused<T, KCH, true, 1>), grid, dim3(256), 0, st, a);
+  else if (vec)
+    hipLaunchKernelGGL((k_train_fused<T, KCH, true, VW>), grid, dim3(256), 0, st, a);
+  else if (one_byte)
+    hipLaunchKernelGGL((k_train_fused<T, KCH, false, 1>), grid, dim3(256), 0, st, a);
   else
-    hipLaunchKernelGGL((k_train_fused<T, KCH, false>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((k_train_fused<T, KCH, false, VW>), grid, dim3(256), 0, st, a);
   SB_LAUNCH_CHECK();
   return 0;
 }
