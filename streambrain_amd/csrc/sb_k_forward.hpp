@@ -8,8 +8,8 @@
 //   B = W : lane (p,q) loads VW consecutive columns of W row k           -> VW column blocks
 // so one 16-byte load of x and VW*NG 16-byte loads of W feed VW*VW*NG MFMAs.  Column block c of group
 // g holds columns j0 + g*16*VW + VW*p + c (interleaved), which makes every result vector
-// {c = 0..VW-1} VW consecutive columns.  Partial tiles are summed through LDS in a fixed tree order,
-// then 16 threads per batch row add the bias and, when FUSE, do the softmax.
+// {c = 0..VW-1} VW consecutive columns.  Partial tiles are summed through LDS in a fixed order, then
+// 16 threads per batch row add the bias and, when FUSE, do the softmax.
 //
 // Tile order: workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  The kernel
 // renumbers them so that one XCD gets a contiguous run of tiles, batch tiles of the same column tile
@@ -17,6 +17,11 @@
 // its workgroups through that XCD's L2.
 #pragma once
 #include "sb_common.hpp"
+
+// Hook for phase timing in development builds; expands to nothing in the library.
+#ifndef SB_PHASE_MARK
+#define SB_PHASE_MARK(n)
+#endif
 
 namespace sb {
 
@@ -34,8 +39,11 @@ struct ForwardArgs {
 // Unguarded 16-byte loads of the main loop: rows / columns outside the matrix are redirected to a valid
 // address (their products land in accumulator rows / columns that are never stored), so the loop body
 // is loads + MFMAs + pointer bumps only.  The last, partial K chunk takes the guarded path.
+// One workgroup per CU is all the tiling provides at small batch sizes, so the register allocator is told
+// to aim for NWAVES/4 wavefronts per SIMD and spend the registers on loads in flight instead.
 template <typename T, int NG, bool FUSE, bool VEC, int NWAVES>
-__global__ __launch_bounds__(64 * NWAVES) void k_forward(ForwardArgs<T> a) {
+__global__ __launch_bounds__(64 * NWAVES) __attribute__((amdgpu_waves_per_eu(NWAVES / 4, NWAVES / 4)))
+void k_forward(ForwardArgs<T> a) {
   constexpr int VW = Real<T>::VW;
   constexpr int GW = 16 * VW;
   constexpr int CP = NG * GW + VW;
@@ -51,7 +59,8 @@ __global__ __launch_bounds__(64 * NWAVES) void k_forward(ForwardArgs<T> a) {
   if (tile >= ntiles) return;  // whole workgroup, before any barrier
   const long ct = tile / a.batch_tiles, bt = tile % a.batch_tiles;
 
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, p = lane & 15, q = lane >> 4;
+  const int tid = threadIdx.x, lane = tid & 63, p = lane & 15, q = lane >> 4;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, in a scalar register: uniform branches
   const long b0 = bt * 16;
   const long j0 = FUSE ? ct * a.Mc : ct * (NG * GW);
   const long jend = FUSE ? j0 + a.Mc : (j0 + NG * GW < a.M ? j0 + NG * GW : a.M);
@@ -64,8 +73,10 @@ __global__ __launch_bounds__(64 * NWAVES) void k_forward(ForwardArgs<T> a) {
 #pragma unroll
     for (int c = 0; c < VW; c++) acc[g][c] = acc_t{0, 0, 0, 0};
 
-  T xa[VW], xb[VW];
-  T wa[VW][NG][VW], wb[VW][NG][VW];
+  // ring of D chunk buffers: D-1 chunks of loads are in flight while one is being multiplied
+  constexpr int D = NG <= 2 ? 3 : 2;
+  T xr[D][VW];
+  T wr[D][VW][NG][VW];
 
   auto compute = [&](const T(&xi)[VW], const T(&wi)[VW][NG][VW]) {
 #pragma unroll
@@ -89,6 +100,7 @@ __global__ __launch_bounds__(64 * NWAVES) void k_forward(ForwardArgs<T> a) {
   };
 
   const long nfull = a.N / KC;  // chunks with all KC reduction indices inside the matrix
+  SB_PHASE_MARK(0);
   if (a.dbg & 1) {
   } else if (VEC) {
     // per-lane pointers of chunk `w`; every later chunk of this wavefront is NWAVES chunks further on
@@ -105,11 +117,15 @@ __global__ __launch_bounds__(64 * NWAVES) void k_forward(ForwardArgs<T> a) {
       }
     const long xstep = (long)NWAVES * KC;
     const long wstep = (long)NWAVES * KC * a.M;
-    auto load_fast = [&](T(&xo)[VW], T(&wo)[VW][NG][VW]) {
+    // Chunks w, w + NWAVES, ... < nfull: n of them for this wavefront.  The loop is branch-free: a load
+    // past the last chunk re-reads the last chunk (its pointers stop advancing) and is never used, so
+    // the compiler can keep exact wait counts and D-1 chunks really are in flight.
+    const long n = w < nfull ? (nfull - 1 - w) / NWAVES + 1 : 0;
+    auto load_next = [&](T(&xo)[VW], T(&wo)[VW][NG][VW], bool advance) {
       const vec_t xv = *reinterpret_cast<const vec_t *>(xp);
 #pragma unroll
       for (int e = 0; e < VW; e++) xo[e] = xv[e];
-      xp += xstep;
+      xp += advance ? xstep : 0;
 #pragma unroll
       for (int s = 0; s < VW; s++)
 #pragma unroll
@@ -117,33 +133,39 @@ __global__ __launch_bounds__(64 * NWAVES) void k_forward(ForwardArgs<T> a) {
           const vec_t wv = *reinterpret_cast<const vec_t *>(wp[s][g]);
 #pragma unroll
           for (int e = 0; e < VW; e++) wo[s][g][e] = wv[e];
-          wp[s][g] += wstep;
+          wp[s][g] += advance ? wstep : 0;
         }
     };
-    // chunks w, w + NWAVES, ... < nfull, two per iteration with one chunk of loads in flight
-    long kc = w;
-    if (kc < nfull) load_fast(xa, wa);
-    while (kc < nfull) {
-      const bool more1 = kc + NWAVES < nfull;
-      if (more1) load_fast(xb, wb);
-      compute(xa, wa);
-      if (!more1) break;
-      const bool more2 = kc + 2 * NWAVES < nfull;
-      if (more2) load_fast(xa, wa);
-      compute(xb, wb);
-      if (!more2) break;
-      kc += 2 * NWAVES;
+    if (n > 0) {
+#pragma unroll
+      for (int u = 0; u < D - 1; u++) load_next(xr[u], wr[u], u + 1 < n);  // chunks 0 .. D-2
+      __builtin_amdgcn_sched_barrier(0);
+      long i = 0;
+      for (; i + D <= n; i += D) {
+#pragma unroll
+        for (int u = 0; u < D; u++) {
+          // the scheduling fences keep the loads where they are written: the compiler's latency model
+          // would otherwise sink them to just ahead of their use, far too late for HBM or L2
+          load_next(xr[(u + D - 1) % D], wr[(u + D - 1) % D], i + u + D < n);  // chunk i + u + D - 1
+          __builtin_amdgcn_sched_barrier(0);
+          compute(xr[u], wr[u]);                                              // chunk i + u
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < D - 1; u++)
+        if (i + u < n) compute(xr[u], wr[u]);
     }
     // partial last chunk (N % KC != 0): one wavefront takes it through the guarded path
     if (nfull * KC < a.N && w == (int)(nfull % NWAVES)) {
-      load_guarded(nfull, xa, wa);
-      compute(xa, wa);
+      load_guarded(nfull, xr[0], wr[0]);
+      compute(xr[0], wr[0]);
     }
   } else {
     const long nchunks = (a.N + KC - 1) / KC;
     for (long kc = w; kc < nchunks; kc += NWAVES) {
-      load_guarded(kc, xa, wa);
-      compute(xa, wa);
+      load_guarded(kc, xr[0], wr[0]);
+      compute(xr[0], wr[0]);
     }
   }
 
@@ -151,37 +173,14 @@ __global__ __launch_bounds__(64 * NWAVES) void k_forward(ForwardArgs<T> a) {
     if (acc[0][0][0] == T(12345.678)) a.act[0] = acc[0][0][0];
     return;
   }
-  // ---- cross-wavefront sum through LDS, halving the number of live partials each round:
-  //      wavefront w + half stores, wavefront w < half adds.  Fixed order => deterministic.
-#pragma unroll
-  for (int half = NWAVES / 2; half >= 1; half >>= 1) {
-    if (w >= half && w < 2 * half) {
-#pragma unroll
-      for (int g = 0; g < NG; g++)
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-          vec_t t;
-#pragma unroll
-          for (int c = 0; c < VW; c++) t[c] = acc[g][c][v];
-          *reinterpret_cast<vec_t *>(&red[w - half][Real<T>::acc_row(q, v)][g * GW + VW * p]) = t;
-        }
-    }
-    __syncthreads();
-    if (w < half) {
-#pragma unroll
-      for (int g = 0; g < NG; g++)
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-          const vec_t t =
-              *reinterpret_cast<const vec_t *>(&red[w][Real<T>::acc_row(q, v)][g * GW + VW * p]);
-#pragma unroll
-          for (int c = 0; c < VW; c++) acc[g][c][v] += t[c];
-        }
-    }
-    __syncthreads();
-  }
-  // wavefront 0 now holds the complete tile; publish it for the row-wise epilogue
-  if (w == 0) {
+  SB_PHASE_MARK(1);
+  // ---- cross-wavefront sum through LDS in a fixed order (deterministic): the upper half of the
+  // wavefronts hands its partial tiles over, the lower half adds them to its own and publishes the
+  // sums (each lane rewrites exactly the elements it has just read, so no barrier is needed between
+  // the two); the row-wise epilogue then adds up the HALF published tiles.
+  constexpr int HALF = NWAVES / 2;
+  static_assert(NWAVES >= 2 && (NWAVES & (NWAVES - 1)) == 0, "a power of two, at least 2 wavefronts");
+  if (w >= HALF) {
 #pragma unroll
     for (int g = 0; g < NG; g++)
 #pragma unroll
@@ -189,11 +188,25 @@ __global__ __launch_bounds__(64 * NWAVES) void k_forward(ForwardArgs<T> a) {
         vec_t t;
 #pragma unroll
         for (int c = 0; c < VW; c++) t[c] = acc[g][c][v];
-        *reinterpret_cast<vec_t *>(&red[0][Real<T>::acc_row(q, v)][g * GW + VW * p]) = t;
+        *reinterpret_cast<vec_t *>(&red[w - HALF][Real<T>::acc_row(q, v)][g * GW + VW * p]) = t;
+      }
+  }
+  __syncthreads();
+  if (w < HALF) {
+#pragma unroll
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        vec_t *slot = reinterpret_cast<vec_t *>(&red[w][Real<T>::acc_row(q, v)][g * GW + VW * p]);
+        vec_t t = *slot;
+#pragma unroll
+        for (int c = 0; c < VW; c++) t[c] += acc[g][c][v];
+        *slot = t;
       }
   }
   __syncthreads();
 
+  SB_PHASE_MARK(2);
   // ---- bias (+ softmax): 16 threads per batch row (256 threads), thread handles columns l16 + 16 t
   if (tid >= 256) return;
   const int row = tid >> 4, l16 = tid & 15;
@@ -206,7 +219,10 @@ __global__ __launch_bounds__(64 * NWAVES) void k_forward(ForwardArgs<T> a) {
     const long col = l16 + 16 * t;
     vals[t] = T(0);
     if (col < ncol) {
-      vals[t] = red[0][row][col] + a.bias[j0 + col];
+      T sum = red[0][row][col];
+#pragma unroll
+      for (int h = 1; h < HALF; h++) sum += red[h][row][col];
+      vals[t] = sum + a.bias[j0 + col];
       mx = vals[t] > mx ? vals[t] : mx;
     }
   }
@@ -238,6 +254,7 @@ __global__ __launch_bounds__(64 * NWAVES) void k_forward(ForwardArgs<T> a) {
       if (col < ncol) out[col] = vals[t];
     }
   }
+  SB_PHASE_MARK(3);
 }
 
 }  // namespace sb

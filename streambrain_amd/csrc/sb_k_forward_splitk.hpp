@@ -21,6 +21,11 @@
 
 #include "sb_common.hpp"
 
+// Hook for phase timing in development builds; expands to nothing in the library.
+#ifndef SB_PHASE_MARK
+#define SB_PHASE_MARK(n)
+#endif
+
 namespace sb {
 
 template <typename T>
@@ -139,9 +144,11 @@ __global__ __launch_bounds__(512) void k_forward_splitk(ForwardSplitArgs<T> a) {
   };
 #pragma unroll
   for (int u = 0; u < PF; u++) load_chunk(c0 + u, wreg[u], xreg[u]);
+  SB_PHASE_MARK(0);
   store_w_chunk(0, wreg[0]);
   store_w_chunk(1, wreg[1]);
   __syncthreads();
+  SB_PHASE_MARK(2);
   read_lds(0, wvA);
   long c = (a.dbg & 1) ? c1 : c0;
   for (; c + PF <= c1; c += PF) {
@@ -155,6 +162,7 @@ __global__ __launch_bounds__(512) void k_forward_splitk(ForwardSplitArgs<T> a) {
   if (c + 1 < c1) step(std::integral_constant<int, 1>{}, c + 1);
   if (c + 2 < c1) step(std::integral_constant<int, 2>{}, c + 2);
 
+  SB_PHASE_MARK(1);
   if (a.dbg & 2) {
     if (acc[0][0][0] == T(12345.678)) a.part[0] = acc[0][0][0];
     return;
@@ -172,6 +180,7 @@ __global__ __launch_bounds__(512) void k_forward_splitk(ForwardSplitArgs<T> a) {
         store_vw<T, VEC>(t, a.part + (ks * a.B + brow) * a.M + j0, (long)g * GW + VW * p, a.Mc);
       }
     }
+  SB_PHASE_MARK(3);
 }
 
 // One wavefront per (batch row, hypercolumn).
