@@ -269,7 +269,7 @@ def main():
     run.evaluate(xt, yt)
     ev_dt = time.perf_counter() - t2
     n, m = 2 * N_PIXELS, H * MC
-    tw = prof.get("train_fused") or prof.get("trace_weights") or {"avg_us": float("nan")}
+    tw = prof.get("train_fused") or {"avg_us": float("nan")}
     alg_bytes = 3 * 4 * n * m  # read Cij, write Cij, write W: 12 bytes per synapse
     achieved = alg_bytes / (tw["avg_us"] * 1e-6) / 1e9
     fwd = prof.get("forward", {"avg_us": float("nan")})

@@ -33,7 +33,6 @@ struct ForwardArgs {
   const T *bias;
   long B, N, M, Mc;
   long col_tiles, batch_tiles;
-  int dbg;  // profiling experiments: bit0 skip the K loop, bit1 leave before the epilogue
 };
 
 // Unguarded 16-byte loads of the main loop: rows / columns outside the matrix are redirected to a valid
@@ -101,8 +100,7 @@ void k_forward(ForwardArgs<T> a) {
 
   const long nfull = a.N / KC;  // chunks with all KC reduction indices inside the matrix
   SB_PHASE_MARK(0);
-  if (a.dbg & 1) {
-  } else if (VEC) {
+  if (VEC) {
     // per-lane pointers of chunk `w`; every later chunk of this wavefront is NWAVES chunks further on
     const long rowc = row_ok ? b0 + p : a.B - 1;
     const T *xp = a.x + rowc * a.N + (long)w * KC + VW * q;
@@ -169,10 +167,6 @@ void k_forward(ForwardArgs<T> a) {
     }
   }
 
-  if (a.dbg & 2) {
-    if (acc[0][0][0] == T(12345.678)) a.act[0] = acc[0][0][0];
-    return;
-  }
   SB_PHASE_MARK(1);
   // ---- cross-wavefront sum through LDS in a fixed order (deterministic): the upper half of the
   // wavefronts hands its partial tiles over, the lower half adds them to its own and publishes the
@@ -214,17 +208,20 @@ void k_forward(ForwardArgs<T> a) {
   constexpr int PER = NG * VW;
   T vals[PER];
   T mx = -INFINITY;
+  T bv[PER];
+#pragma unroll
+  for (int t = 0; t < PER; t++) {  // branch-free, so the loads are in flight together
+    const long col = l16 + 16 * t;
+    bv[t] = a.bias[j0 + (col < ncol ? col : 0)];
+  }
 #pragma unroll
   for (int t = 0; t < PER; t++) {
     const long col = l16 + 16 * t;
-    vals[t] = T(0);
-    if (col < ncol) {
-      T sum = red[0][row][col];
+    T sum = red[0][row][col < ncol ? col : 0];
 #pragma unroll
-      for (int h = 1; h < HALF; h++) sum += red[h][row][col];
-      vals[t] = sum + a.bias[j0 + col];
-      mx = vals[t] > mx ? vals[t] : mx;
-    }
+    for (int h = 1; h < HALF; h++) sum += red[h][row][col < ncol ? col : 0];
+    vals[t] = col < ncol ? sum + bv[t] : T(0);
+    mx = (col < ncol && vals[t] > mx) ? vals[t] : mx;
   }
   if (FUSE) {
 #pragma unroll

@@ -8,21 +8,25 @@
 //   bias/kbi <- update_bias_regularized(Cj)                (plastic layers)
 // all from the NEW traces, as the reference's fused loop does.
 //
-// A workgroup (256 threads, 4 wavefronts) owns a 64 x 64 tile of Cij.
-//   1. It requests its Cij tile right away (16-byte vectors, 256 contiguous bytes per 16 threads), so
-//      the HBM latency of the stream hides behind everything that follows.
-//   2. Per chunk of KCH batch rows it stages x[:, i-tile] and y[:, j-tile] in LDS with all loads in
-//      flight at once.  x and y are "k-major" in memory, which is the 16x16x4 MFMA operand layout, so
-//      staging is a plain copy and each wavefront feeds its 32 x 32 sub-tile (2 x 2 MFMA blocks) with
-//      two 8-byte LDS reads per K step of 4.
-//   3. From the same LDS slabs, 32 lanes of each wavefront add up one column each of x (resp. y) in
+// A workgroup (256 threads, 4 wavefronts) owns a 64 x 64 tile of Cij; 16 KiB of LDS and at most 96
+// registers per thread let five workgroups share a CU, so the 1175 tiles of a 1568 x 3000 layer are
+// all resident at once.
+//   1. Per chunk of KCH batch rows it stages x[:, i-tile] and y[:, j-tile] in LDS.  x and y are
+//      "k-major" in memory, which is the 16x16x4 MFMA operand layout, so staging is a plain copy and
+//      each wavefront feeds its 32 x 32 sub-tile (2 x 2 MFMA blocks) with two 8-byte LDS reads per K
+//      step of 4.  The global loads of chunk c+1 are issued before chunk c is consumed.
+//   2. From the same LDS slabs, 32 lanes of each wavefront add up one column each of x (resp. y) in
 //      batch order b = 0..B-1 without FMA contraction: the reference's summation order, so Ci, Cj and
 //      kbi stay bit-exact against a strict-IEEE build of it.  Every tile needs Ci for its rows and Cj
 //      for its columns, so every workgroup recomputes them from the OLD traces (a tile row shares x,
 //      a tile column shares y: same inputs, same order, same bits).  The old traces are read from
 //      Ci/Cj and the new ones written to Ci_next/Cj_next by the tiles of the first tile column / row:
 //      no workgroup ever reads a value another one is writing.
-//   4. The accumulators go through LDS into a row-major layout; each thread then finishes 4 consecutive
+//   3. Global loads return in issue order, so the Cij tile (HBM latency) is requested only while the
+//      second-to-last chunk is being multiplied: the MFMA loop never waits for it, and it has arrived
+//      by the time the epilogue needs it.  All loads are branch-free (clamped addresses): a guarded
+//      load makes the compiler wait for every outstanding load at the join.
+//   4. The accumulators go through LDS into a row-major layout; each thread then finishes VW consecutive
 //      columns of 4 rows: decay + clamp, weight, mask, one 16-byte store each to Cij and W.
 #pragma once
 #include <type_traits>

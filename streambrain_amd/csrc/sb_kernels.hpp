@@ -33,24 +33,7 @@ __global__ __launch_bounds__(256) void k_softmax(T *act, long groups, long Mc) {
   for (long c = lane; c < Mc; c += 64) v[c] = v[c] / sum;
 }
 
-// =====================================================================================================
-// Ci / Cj moving averages (+ bias of a plastic layer)                   omp.cc:106-156, 222-246
-// One thread per trace element; the batch sum runs b = 0..B-1 in REAL without FMA contraction, then
-// /B, *taupdt, C*(1-taupdt) + tmp, max(0, .) -- the reference's order, so Ci and Cj are bit-exact
-// against a strict-IEEE build of it.
-// =====================================================================================================
-template <typename T>
-struct CountersArgs {
-  const T *x;  // [B,N]
-  const T *y;  // [B,M]
-  T *Ci, *Cj;
-  long B, N, M;
-  T tau, omt, fB;
-  int bias_mode;  // 0: leave bias alone; 1: update_bias_regularized on the fresh Cj
-  T *bias, *kbi;
-  T cthr, khalf, pmin, taubdt;
-};
-
+// update_bias_regularized for one unit (omp.cc:222-246); kbi is updated in place.
 template <typename T>
 __device__ __forceinline__ T bias_regularized(T pj, T &kbi, T cthr, T khalf, T pmin, T taubdt) {
   using R = Real<T>;
@@ -332,5 +315,4 @@ __global__ __launch_bounds__(256) void k_fill(T *dst, T value, size_t n) {
 }  // namespace sb
 
 #include "sb_k_forward.hpp"
-#include "sb_k_traces.hpp"
 #include "sb_k_mask_swap.hpp"

@@ -30,7 +30,7 @@ struct TraceScalars {
 // Per-kernel timing: when profiling is on (sb_profile_start), every launcher brackets its launches
 // with a pair of HIP events on the launch stream; sb_profile_stop sums the elapsed times per kernel.
 enum KernelId {
-  K_FORWARD = 0, K_SOFTMAX, K_COUNTERS, K_TRACE_WEIGHTS, K_UPDATE_BIAS, K_UPDATE_BIAS_REG, K_MASK_SCORES,
+  K_FORWARD = 0, K_SOFTMAX, K_UPDATE_BIAS, K_UPDATE_BIAS_REG, K_MASK_SCORES,
   K_MASK_SWAP, K_MASK_FIX, K_APPLY_MASK, K_ARGMAX, K_GATHER, K_FILL, K_TRAIN_FUSED, K_COUNT
 };
 const char *kernel_name(int id);
@@ -58,27 +58,11 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
     }                                                 \
   } while (0)
 
-// The split-K forward needs scratch for its partial sums: forward_plan says how many elements (0 when
-// the shape does not qualify); launch_forward uses that path when `scratch` is large enough and falls
-// back to the single-kernel forms otherwise.
-struct ForwardPlan {
-  long KS;             // slices of the reduction dimension
-  long scratch_elems;  // KS * B * M, or 0
-};
-template <typename T>
-ForwardPlan forward_plan(long B, long N, long H, long Mc);
 template <typename T>
 int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias, long B, long N,
-                   long H, long Mc, bool softmax, T *scratch, size_t scratch_elems);
+                   long H, long Mc, bool softmax);
 template <typename T>
 int launch_softmax(hipStream_t st, T *act, long B, long H, long Mc);
-template <typename T>
-int launch_counters(hipStream_t st, const T *x, const T *y, T *Ci, T *Cj, long B, long N, long M,
-                    T taupdt, int bias_mode, T *bias, T *kbi, T cthr, T khalf, T pmin, T taubdt);
-template <typename T>
-int launch_trace_weights(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci,
-                         const T *Cj, const uint8_t *wmask, long B, long N, long H, long Mc, T taupdt,
-                         T cthr);
 // Fused Ci/Cj/Cij + weights (+ regularised bias when bias_mode == 1, + mask when wmask != nullptr).
 // Reads the old traces from Ci/Cj and writes the new ones to Ci_next/Cj_next (distinct buffers).
 template <typename T>

@@ -3,7 +3,6 @@
 #pragma once
 #include "sb_kernels.hpp"
 #include "sb_k_train.hpp"
-#include "sb_k_forward_splitk.hpp"
 #include "sb_launch.hpp"
 
 #include <cstdlib>
@@ -26,20 +25,6 @@ static int forward_variant(hipStream_t st, ForwardArgs<T> a, bool vec) {
     set_error("launch_forward: too many tiles for one launch");
     return -1;
   }
-  static const int waves_env = [] {
-    const char *e = getenv("SB_FWD_WAVES");
-    return e ? atoi(e) : 0;
-  }();
-  if constexpr (NG <= 2) {
-    if (waves_env == 16) {
-      if (vec)
-        hipLaunchKernelGGL((k_forward<T, NG, FUSE, true, 16>), dim3((unsigned)grid), dim3(1024), 0, st, a);
-      else
-        hipLaunchKernelGGL((k_forward<T, NG, FUSE, false, 16>), dim3((unsigned)grid), dim3(1024), 0, st, a);
-      SB_LAUNCH_CHECK();
-      return 0;
-    }
-  }
   if (vec)
     hipLaunchKernelGGL((k_forward<T, NG, FUSE, true, 8>), dim3((unsigned)grid), dim3(512), 0, st, a);
   else
@@ -61,74 +46,17 @@ static inline int device_cu_count() {
 }
 
 template <typename T>
-ForwardPlan forward_plan(long B, long N, long H, long Mc) {
-  constexpr int VW = Real<T>::VW;
-  ForwardPlan plan{0, 0};
-  if (cdiv(Mc, 16 * VW) > 8 || B <= 0 || N <= 0 || H <= 0) return plan;
-  const long chunks = cdiv(N, 4 * VW);
-  const long tiles = cdiv(B, 128) * H;
-  long ks = device_cu_count() / tiles;  // about one workgroup per CU
-  static const int ks_env = [] {
-    const char *e = getenv("SB_FWD_KS");
-    return e ? atoi(e) : 0;
-  }();
-  if (ks_env > 0) ks = ks_env;
-  if (ks < 1) ks = 1;
-  if (ks > chunks) ks = chunks;
-  plan.KS = ks;
-  plan.scratch_elems = ks * B * H * Mc;
-  return plan;
-}
-
-template <typename T>
 int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias, long B, long N,
-                   long H, long Mc, bool softmax, T *scratch, size_t scratch_elems) {
+                   long H, long Mc, bool softmax) {
   constexpr int VW = Real<T>::VW;
   constexpr int GW = 16 * VW;
   SB_REQUIRE(act && x && W && bias, "null pointer");
   SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");
   const long M = H * Mc;
   SB_REQUIRE(M < (1L << 31) && N < (1L << 31), "dimension too large");
-  ForwardArgs<T> a{act, x, W, bias, B, N, M, Mc, 0, cdiv(B, 16), 0};
-  {
-    const char *e = getenv("SB_DBG");
-    a.dbg = e ? atoi(e) : 0;
-  }
+  ForwardArgs<T> a{act, x, W, bias, B, N, M, Mc, 0, cdiv(B, 16)};
   const bool base_vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(W);
   const long need = cdiv(Mc, GW);
-  // split-K path: needs the partial-sum scratch and a hypercolumn that fits one staged tile
-  const ForwardPlan plan = forward_plan<T>(B, N, H, Mc);
-  // measured slower than the single-kernel form at the MNIST shape (two launches, partial-sum round
-  // trip); kept selectable for shapes with many batch rows per hypercolumn
-  static const bool no_splitk = getenv("SB_FWD_SPLIT") == nullptr;
-  if (softmax && plan.scratch_elems > 0 && scratch && scratch_elems >= (size_t)plan.scratch_elems &&
-      !no_splitk) {
-    ForwardSplitArgs<T> sa{scratch, x, W, B, N, M, H, Mc, plan.KS, cdiv(N, 4 * VW), a.dbg};
-    const bool vec = base_vec && (Mc % VW == 0) && aligned16(scratch);
-    const long grid = cdiv(B, 128) * H * plan.KS;
-    SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
-    {
-      ProfScope prof_(st, K_FORWARD);
-#define SB_FWD_SPLIT(NG_)                                                                            \
-  do {                                                                                               \
-    if (vec)                                                                                         \
-      hipLaunchKernelGGL((k_forward_splitk<T, NG_, true>), dim3((unsigned)grid), dim3(512), 0, st, sa); \
-    else                                                                                             \
-      hipLaunchKernelGGL((k_forward_splitk<T, NG_, false>), dim3((unsigned)grid), dim3(512), 0, st, sa); \
-  } while (0)
-      if (need <= 1) SB_FWD_SPLIT(1);
-      else if (need <= 2) SB_FWD_SPLIT(2);
-      else if (need <= 4) SB_FWD_SPLIT(4);
-      else SB_FWD_SPLIT(8);
-#undef SB_FWD_SPLIT
-      SB_LAUNCH_CHECK();
-    }
-    ProfScope prof_(st, K_SOFTMAX);
-    hipLaunchKernelGGL((k_forward_finish<T>), dim3((unsigned)cdiv(B * H, 4)), dim3(256), 0, st, act,
-                       (const T *)scratch, bias, B, M, H, Mc, plan.KS, 1);
-    SB_LAUNCH_CHECK();
-    return 0;
-  }
   const long max_fused = sizeof(T) == 4 ? 4 : 7;
   if (softmax && need <= max_fused) {
     const bool vec = base_vec && (Mc % VW == 0);
@@ -158,92 +86,7 @@ int launch_softmax(hipStream_t st, T *act, long B, long H, long Mc) {
   return 0;
 }
 
-// ------------------------------------------------------------------------------------------ counters
-template <typename T>
-int launch_counters(hipStream_t st, const T *x, const T *y, T *Ci, T *Cj, long B, long N, long M,
-                    T taupdt, int bias_mode, T *bias, T *kbi, T cthr, T khalf, T pmin, T taubdt) {
-  SB_REQUIRE(x && y && Ci && Cj, "null pointer");
-  SB_REQUIRE(B > 0 && N > 0 && M > 0, "sizes must be positive");
-  SB_REQUIRE(bias_mode == 0 || (bias && kbi), "bias update needs bias and kbi");
-  CountersArgs<T> a;
-  a.x = x; a.y = y; a.Ci = Ci; a.Cj = Cj; a.B = B; a.N = N; a.M = M;
-  a.tau = taupdt; a.omt = (T)(1.0 - (double)taupdt); a.fB = (T)B;
-  a.bias_mode = bias_mode; a.bias = bias; a.kbi = kbi;
-  a.cthr = cthr; a.khalf = khalf; a.pmin = pmin; a.taubdt = taubdt;
-  ProfScope prof_(st, K_COUNTERS);
-  hipLaunchKernelGGL((k_counters<T>), dim3((unsigned)(cdiv(N, 64) + cdiv(M, 64))), dim3(256), 0, st, a);
-  SB_LAUNCH_CHECK();
-  return 0;
-}
-
-// ------------------------------------------------------------------------------------- trace + weights
-template <typename T, int XW, int YW, int RX, int RY>
-static int trace_variant(hipStream_t st, const TraceArgs<T> &a, bool vec) {
-  ProfScope prof_(st, K_TRACE_WEIGHTS);
-  dim3 grid((unsigned)cdiv(a.M, 2 * RY * 16 * YW), (unsigned)cdiv(a.N, 2 * RX * 16 * XW));
-  if (grid.y > 65535) {
-    set_error("launch_trace_weights: in_features too large for one launch");
-    return -1;
-  }
-  if (vec)
-    hipLaunchKernelGGL((k_trace_weights<T, XW, YW, RX, RY, true, true>), grid, dim3(256), 0, st, a);
-  else
-    hipLaunchKernelGGL((k_trace_weights<T, XW, YW, RX, RY, false, true>), grid, dim3(256), 0, st, a);
-  SB_LAUNCH_CHECK();
-  return 0;
-}
-
-static inline int dbg_flags() {
-  static const int v = [] {
-    const char *e = getenv("SB_DBG");
-    return e ? atoi(e) : 0;
-  }();
-  return v;
-}
-
-static inline int trace_tile_choice() {
-  static const int v = [] {
-    const char *e = getenv("SB_TRACE_TILE");
-    return e ? atoi(e) : 0;
-  }();
-  return v;
-}
-
-template <typename T>
-int launch_trace_weights(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci,
-                         const T *Cj, const uint8_t *wmask, long B, long N, long H, long Mc, T taupdt,
-                         T cthr) {
-  constexpr int VW = Real<T>::VW;
-  SB_REQUIRE(x && y && Cij && W && Ci && Cj, "null pointer");
-  SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");
-  const long M = H * Mc;
-  SB_REQUIRE(M < (1L << 31) && N < (1L << 31), "dimension too large");
-  const TraceScalars<T> s = TraceScalars<T>::from(taupdt, cthr);
-  TraceArgs<T> a;
-  a.x = x; a.y = y; a.Cij = Cij; a.W = W; a.Ci = Ci; a.Cj = Cj; a.wmask = wmask;
-  a.B = B; a.N = N; a.M = M; a.H = H; a.Mc = Mc;
-  a.tau = s.tau; a.omt = s.omt; a.invB = (T)1 / (T)B; a.cthr = s.cthr; a.cthr4 = s.cthr4;
-  a.dbg = dbg_flags();
-  const bool vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(y) && aligned16(Cij) &&
-                   aligned16(W);
-  if constexpr (sizeof(T) == 4) {
-    switch (trace_tile_choice()) {
-      case 1: return trace_variant<T, 2, 4, 1, 1>(st, a, vec);   // 32 x 64
-      case 2: return trace_variant<T, 2, 2, 1, 1>(st, a, vec);   // 32 x 32
-      case 3: return trace_variant<T, 1, 4, 1, 1>(st, a, vec);   // 16 x 64
-      case 4: return trace_variant<T, 4, 2, 1, 1>(st, a, vec);   // 64 x 32
-      case 5: return trace_variant<T, 1, 4, 2, 1>(st, a, vec);   // 32 x 64, x as two 4-byte loads
-      default: return trace_variant<T, 4, 4, 1, 1>(st, a, vec);  // 64 x 64
-    }
-  } else {
-    return trace_variant<T, 2, 2, 1, 2>(st, a, vec);  // 32 x 64
-  }
-}
-
 // ------------------------------------------------------------------------------------- fused training
-#ifndef SB_TRAIN_KCH
-#define SB_TRAIN_KCH 32
-#endif
 template <typename T>
 int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci, const T *Cj,
                        T *Ci_next, T *Cj_next, const uint8_t *wmask, int bias_mode, T *bias, T *kbi,
@@ -267,9 +110,8 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   const bool vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(y) && aligned16(Cij) &&
                    aligned16(W);
   const dim3 grid((unsigned)(a.tiles_i * a.tiles_j));
-  SB_REQUIRE(M < (1L << 31), "more than 2^31 output units");
-  // batch rows staged per chunk
-  constexpr int KCH = SB_TRAIN_KCH;
+  // batch rows staged per chunk: 16 KiB of LDS per workgroup, so five workgroups share a CU
+  constexpr int KCH = 32;
   const bool one_byte = Mc % VW == 0;  // every vector of VW columns lies inside one hypercolumn
   ProfScope prof_(st, K_TRAIN_FUSED);
   if (vec && one_byte)
@@ -405,14 +247,9 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
 }
 
 #define SB_INSTANTIATE_LAUNCHERS(T)                                                                   \
-  template ForwardPlan forward_plan<T>(long, long, long, long);                                       \
   template int launch_forward<T>(hipStream_t, T *, const T *, const T *, const T *, long, long, long, \
-                                 long, bool, T *, size_t);                                            \
+                                 long, bool);                                                         \
   template int launch_softmax<T>(hipStream_t, T *, long, long, long);                                 \
-  template int launch_counters<T>(hipStream_t, const T *, const T *, T *, T *, long, long, long, T,   \
-                                  int, T *, T *, T, T, T, T);                                         \
-  template int launch_trace_weights<T>(hipStream_t, const T *, const T *, T *, T *, const T *,        \
-                                       const T *, const uint8_t *, long, long, long, long, T, T);     \
   template int launch_train_fused<T>(hipStream_t, const T *, const T *, T *, T *, const T *, const T *, \
                                      T *, T *, const uint8_t *, int, T *, T *, long, long, long, long, \
                                      T, T, T, T, T);                                                   \

@@ -35,8 +35,6 @@ struct Context {
   void *trace_next = nullptr;
   long trace_cap = 0;  // elements of 8 bytes
   // partial sums of the split-K forward, shared by every caller (stream order serialises its use)
-  void *fwd_part = nullptr;
-  size_t fwd_cap = 0;  // bytes
 };
 static Context g_ctx;
 static std::mutex g_ctx_mutex;
@@ -54,7 +52,7 @@ static long g_prof_launches[K_COUNT];
 static double g_prof_overhead_ms = 0;  // elapsed time of an empty event bracket
 
 const char *kernel_name(int id) {
-  static const char *names[K_COUNT] = {"forward", "softmax", "counters", "trace_weights", "update_bias",
+  static const char *names[K_COUNT] = {"forward", "softmax", "update_bias",
                                        "update_bias_regularized", "mask_scores", "mask_swap",
                                        "mask_fix_weights", "apply_mask", "argmax", "gather_rows", "fill",
                                        "train_fused"};
@@ -123,31 +121,6 @@ static int ensure_trace_scratch(long elems) {
   return 0;
 }
 
-template <typename T>
-static int forward_scratch(long B, long N, long H, long Mc, T **scratch, size_t *elems) {
-  const ForwardPlan plan = forward_plan<T>(B, N, H, Mc);
-  const size_t bytes = (size_t)plan.scratch_elems * sizeof(T);
-  if (bytes > g_ctx.fwd_cap) {
-    SB_HIP(hipStreamSynchronize(g_ctx.stream));
-    if (g_ctx.fwd_part) SB_HIP(hipFree(g_ctx.fwd_part));
-    g_ctx.fwd_part = nullptr;
-    g_ctx.fwd_cap = 0;
-    SB_HIP(hipMalloc(&g_ctx.fwd_part, bytes));
-    g_ctx.fwd_cap = bytes;
-  }
-  *scratch = (T *)g_ctx.fwd_part;
-  *elems = g_ctx.fwd_cap / sizeof(T);
-  return 0;
-}
-
-static bool use_old_train_path() {
-  static const bool v = [] {
-    const char *e = getenv("SB_TRAIN_PATH");
-    return e && std::string(e) == "old";
-  }();
-  return v;
-}
-
 // Per-kernel entry points keep the reference's in-place contract: the fused kernel writes the new
 // Ci / Cj into scratch, which is then copied over the caller's arrays.
 template <typename T>
@@ -156,12 +129,6 @@ static int train_in_place(const T *x, const T *y, T *Cij, T *W, T *Ci, T *Cj, co
                           T cthr, T khalf, T pmin, T taubdt) {
   hipStream_t st = g_ctx.stream;
   const long M = H * Mc;
-  if (use_old_train_path()) {
-    int rc = launch_counters<T>(st, x, y, Ci, Cj, B, N, M, taupdt, bias_mode, bias, kbi, cthr, khalf,
-                                pmin, taubdt);
-    if (rc) return rc;
-    return launch_trace_weights<T>(st, x, y, Cij, W, Ci, Cj, wmask, B, N, H, Mc, taupdt, cthr);
-  }
   SB_REQUIRE(N > 0 && M > 0, "sizes must be positive");
   int rc = ensure_trace_scratch(N + M);
   if (rc) return rc;
@@ -263,12 +230,8 @@ static int ensure_act(sb_net *net, long rows) {
 
 template <typename T>
 static int layer_forward(const Layer &L, const T *x, long B) {
-  T *scratch = nullptr;
-  size_t elems = 0;
-  int rc = forward_scratch<T>(B, L.N, L.H, L.Mc, &scratch, &elems);
-  if (rc) return rc;
   return launch_forward<T>(g_ctx.stream, (T *)L.act, x, (const T *)L.W, (const T *)L.bias, B, L.N, L.H,
-                           L.Mc, true, scratch, elems);
+                           L.Mc, true);
 }
 
 // One training step of `L` on input x (and on y = its own activation or the labels), in the order of
@@ -280,23 +243,13 @@ static int layer_train_step(Layer &L, const T *x, const T *y, long B, long h) {
   const T tau = (T)L.taupdt;
   const T cthr = (T)(L.taupdt / 2);
   int rc = 0;
-  if (use_old_train_path()) {
-    rc = launch_counters<T>(st, x, y, (T *)L.Ci, (T *)L.Cj, B, L.N, L.M, tau, L.plastic ? 1 : 0,
-                            (T *)L.bias, (T *)L.kbi, cthr, (T)L.khalf, (T)L.pmin, (T)L.taubdt);
-    if (rc) return rc;
-    rc = launch_trace_weights<T>(st, x, y, (T *)L.Cij, (T *)L.W, (const T *)L.Ci, (const T *)L.Cj,
-                                 L.plastic ? L.wmask : nullptr, B, L.N, L.H, L.Mc, tau, cthr);
-  } else {
-    rc = launch_train_fused<T>(st, x, y, (T *)L.Cij, (T *)L.W, (const T *)L.Ci, (const T *)L.Cj,
-                               (T *)L.Ci_alt, (T *)L.Cj_alt, L.plastic ? L.wmask : nullptr,
-                               L.plastic ? 1 : 0, (T *)L.bias, (T *)L.kbi, B, L.N, L.H, L.Mc, tau, cthr,
-                               (T)L.khalf, (T)L.pmin, (T)L.taubdt);
-    if (!rc) {
-      std::swap(L.Ci, L.Ci_alt);
-      std::swap(L.Cj, L.Cj_alt);
-    }
-  }
+  rc = launch_train_fused<T>(st, x, y, (T *)L.Cij, (T *)L.W, (const T *)L.Ci, (const T *)L.Cj,
+                             (T *)L.Ci_alt, (T *)L.Cj_alt, L.plastic ? L.wmask : nullptr,
+                             L.plastic ? 1 : 0, (T *)L.bias, (T *)L.kbi, B, L.N, L.H, L.Mc, tau, cthr,
+                             (T)L.khalf, (T)L.pmin, (T)L.taubdt);
   if (rc) return rc;
+  std::swap(L.Ci, L.Ci_alt);
+  std::swap(L.Cj, L.Cj_alt);
   if (L.plastic && h >= 0) {
     rc = launch_update_mask<T>(st, L.wmask, (const T *)nullptr, (const T *)L.Ci, (const T *)L.Cj,
                                (const T *)L.Cij, cthr, L.N, L.H, L.Mc, h, 16, (T *)L.nom, L.csum);
@@ -515,7 +468,6 @@ int sb_shutdown(void) {
   if (g_ctx.mask_nom) SB_HIP(hipFree(g_ctx.mask_nom));
   if (g_ctx.mask_csum) SB_HIP(hipFree(g_ctx.mask_csum));
   if (g_ctx.trace_next) SB_HIP(hipFree(g_ctx.trace_next));
-  if (g_ctx.fwd_part) SB_HIP(hipFree(g_ctx.fwd_part));
   SB_HIP(hipStreamDestroy(g_ctx.stream));
   g_ctx = Context();
   return 0;
@@ -574,7 +526,7 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
 #define SB_DEFINE_KERNEL_API(SFX, T)                                                                   \
   int sb_update_state_##SFX(T *act, const T *x, const T *W, const T *bias, long B, long N, long M) {   \
     SB_READY();                                                                                        \
-    return launch_forward<T>(g_ctx.stream, act, x, W, bias, B, N, 1, M, false, (T *)nullptr, 0);       \
+    return launch_forward<T>(g_ctx.stream, act, x, W, bias, B, N, 1, M, false);                        \
   }                                                                                                    \
   int sb_softmax_minicolumns_##SFX(T *act, long B, long H, long Mc) {                                  \
     SB_READY();                                                                                        \
@@ -584,11 +536,7 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
                                   long H, long Mc) {                                                   \
     SB_READY();                                                                                        \
     SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");                           \
-    T *scratch = nullptr;                                                                              \
-    size_t elems = 0;                                                                                  \
-    int rc = forward_scratch<T>(B, N, H, Mc, &scratch, &elems);                                        \
-    if (rc) return rc;                                                                                 \
-    return launch_forward<T>(g_ctx.stream, act, x, W, bias, B, N, H, Mc, true, scratch, elems);        \
+    return launch_forward<T>(g_ctx.stream, act, x, W, bias, B, N, H, Mc, true);                        \
   }                                                                                                    \
   int sb_update_weights_##SFX(T *Ci, T *Cj, T *Cij, const T *a_i, const T *a_o, T taupdt, T *W,        \
                               T cthr, long B, long N, long M) {                                        \
