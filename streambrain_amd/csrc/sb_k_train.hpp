@@ -83,13 +83,23 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   T *rci_s = slab + TS * CP, *rcj_s = rci_s + TS;
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, p = lane & 15, q = lane >> 4;
-  const long it = (long)blockIdx.x / a.tiles_j, jt = (long)blockIdx.x % a.tiles_j;
+  // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  Renumbered so that one XCD
+  // gets a contiguous run of tiles in column-major order: a few tile columns, i.e. a few hundred KB of
+  // y plus all of x, instead of all of x and y per L2.
+  const long ntiles = a.tiles_i * a.tiles_j;
+  const long per_xcd = (ntiles + 7) / 8;
+  const long tile = (long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (tile >= ntiles) return;  // whole workgroup, before any barrier
+  const long jt = tile / a.tiles_i, it = tile % a.tiles_i;
   const long i0 = it * TS, j0 = jt * TS;
 
   // thread's share of the tile in row-major order: VW columns of PASSES rows
   const int eg = tid % G, er = tid / G;
   const long ecol = j0 + VW * eg;
 
+#ifdef SB_STAGGER
+  for (int z = 0; z < (int)(blockIdx.x / 256) * SB_STAGGER; z++) __builtin_amdgcn_s_sleep(16);
+#endif
   SB_PHASE_MARK(0);
   // All global loads are branch-free (clamped addresses; what a guard excludes is zeroed or ignored
   // where it is consumed), so they stay in flight together.  Loads return in issue order, hence the

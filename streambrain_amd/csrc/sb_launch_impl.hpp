@@ -106,10 +106,11 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   a.tau = s.tau; a.omt = s.omt; a.fB = (T)B; a.invB = (T)1 / (T)B; a.cthr = s.cthr; a.cthr4 = s.cthr4;
   a.khalf = khalf; a.pmin = pmin; a.taubdt = taubdt;
   a.tiles_i = cdiv(N, 64); a.tiles_j = cdiv(M, 64);
-  SB_REQUIRE(a.tiles_i * a.tiles_j < (1L << 31), "too many tiles for one launch");
+  SB_REQUIRE(a.tiles_i * a.tiles_j < (1L << 31) - 8, "too many tiles for one launch");
   const bool vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(y) && aligned16(Cij) &&
                    aligned16(W);
-  const dim3 grid((unsigned)(a.tiles_i * a.tiles_j));
+  // 8 workgroup ids per round of XCDs; ids beyond the last tile exit at once
+  const dim3 grid((unsigned)(8 * cdiv(a.tiles_i * a.tiles_j, 8)));
   // batch rows staged per chunk: 16 KiB of LDS per workgroup, so five workgroups share a CU
   constexpr int KCH = 32;
   const bool one_byte = Mc % VW == 0;  // every vector of VW columns lies inside one hypercolumn
