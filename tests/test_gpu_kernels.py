@@ -177,6 +177,32 @@ def test_update_mask_ties_and_degenerate_columns(k, oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("N", [24, 700, 3000])
+def test_update_mask_nan_scores(k, oracle, dtype, N):
+    """Rows with Ci = 1 and Cij = Cj give 0 * log(x/0) = NaN nominators.  The reference's sequential
+    `>=` / `<=` scan lets a NaN win only when it is the first candidate of its group; the strict-IEEE
+    oracle restates exactly that, and the GPU reduction has to reproduce it bit for bit."""
+    rng = np.random.default_rng(N)
+    H, Mc = 3, 4
+    wmask, W, Ci, Cj, Cij = _mask_problem(rng, N, H, Mc, dtype, density=0.3)
+    for case in range(6):
+        ci, cij, wm = Ci.copy(), Cij.copy(), wmask.copy()
+        bad = rng.choice(N, size=max(2, N // 10), replace=False)
+        if case % 3 == 1:
+            bad[0] = 0  # a NaN on the very first row
+        if case % 3 == 2:
+            first_active = int(np.flatnonzero(wm[:, 1])[0])
+            bad[0] = first_active  # a NaN on the first active row
+        ci[bad] = 1.0
+        cij[bad, :] = Cj[None, :]
+        trace = {}
+        ref = oracle.update_mask(wm.copy(), W, ci, Cj, cij, 0.01, H, Mc, 1, 16, trace=trace)
+        got = k.update_mask(wm.copy(), W, ci, Cj, cij, 0.01, H, Mc, 1, 16)
+        assert np.array_equal(got, ref), f"case {case}: masks differ in {(got != ref).sum()} entries, " \
+                                         f"swaps {trace['swaps']}"
+
+
+@pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("N,H,Mc", [(1, 1, 1), (13, 4, 5), (1568, 30, 100), (100, 7, 9)])
 def test_apply_mask(k, oracle, dtype, N, H, Mc):
     rng = np.random.default_rng(N)
