@@ -115,6 +115,36 @@ def test_mnist_shape_one_epoch_f32(hb):
     assert cg.tolist() == cr.tolist()
 
 
+def test_dense_hidden_layer_one_epoch_f32(hb):
+    # The hidden layer with an all-ones mask (density 1) trained for one epoch on its own activations,
+    # float32, batch 128, a short last batch: the reference's cpu-runnable single-layer case on fewer
+    # batches (the output layer is only there because fit trains the LAST layer on labels).
+    from oracle import cpu_backend as ob
+    rng = np.random.default_rng(1000)
+    X = synthetic_images(rng, 20 * 128 - 32, 784)
+    Y = one_hot_labels(rng, X.shape[0], 10)
+    nets = []
+    for backend in (hb, ob):
+        net = build_two_layer(backend, 1568, 30, 100, 10, MNIST_HP, np.float32, seed=0, density=1.0)
+        net.fit(X, Y, 128, [(0, 1)])
+        nets.append(net)
+    g, r = nets
+    assert g._layers[0].wmask.all() and r._layers[0].wmask.all()
+    for name in ("Ci", "Cj", "Cij", "weights", "bias", "kbi"):
+        e = rel_err(getattr(g._layers[0], name), getattr(r._layers[0], name))
+        assert e <= 1e-4, f"{name}: {e:.3e}"
+
+
+def test_wide_hidden_layer_f64(hb):
+    # 1568 -> 100 x 100 -> 10 in float64 with batch 512 (one full and one short batch per epoch): the
+    # float64 MFMA path of the trace GEMM and the float64 log / divide of the weight pass.
+    (g, r), (Xt, Yt) = _run_both(hb, np.float64, n_pix=784, H=100, Mc=100, n_out=10, Ns=512 + 96, Nt=64,
+                                 B=512, e1=1, e2=1, hp=MNIST_HP, data_seed=1002)
+    assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
+    _compare_states(g, r, 1e-11)
+    assert np.array_equal(g.predict(Xt, 512), r.predict(Xt, 512))
+
+
 def test_mnist_shape_rewiring_epoch_f32(hb):
     # Second epoch, with rewiring (31 // 31 = 1: hypercolumns rewire on steps 0..29).  Over a float32
     # TRAJECTORY mask equality is not well defined: each swap compares scores that are sums of
