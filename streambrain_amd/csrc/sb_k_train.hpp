@@ -197,17 +197,25 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
       }
     }
 
-    // K loop: per step of 4 batch rows, lane (p,q) feeds row 4s+q of the slabs
+    // K loop: per step of 4 batch rows, lane (p,q) feeds row 4s+q of the slabs.  The operands of step
+    // s+1 are read from LDS before the MFMAs of step s are issued (the fences keep that order).
     const T *xa = xs + q * TS + iw + 2 * p;
     const T *ya = ys + q * TS + jw + 2 * p;
-#pragma unroll 8
+    T xo[2][2], yo[2][2];
+    xo[0][0] = xa[0], xo[0][1] = xa[1], yo[0][0] = ya[0], yo[0][1] = ya[1];
+#pragma unroll
     for (int s = 0; s < KCH / 4; s++) {
-      const T x0 = xa[s * 4 * TS], x1 = xa[s * 4 * TS + 1];
-      const T y0 = ya[s * 4 * TS], y1 = ya[s * 4 * TS + 1];
-      acc[0][0] = R::mfma(x0, y0, acc[0][0]);
-      acc[0][1] = R::mfma(x0, y1, acc[0][1]);
-      acc[1][0] = R::mfma(x1, y0, acc[1][0]);
-      acc[1][1] = R::mfma(x1, y1, acc[1][1]);
+      const int cur = s & 1, nxt = cur ^ 1;
+      if (s + 1 < KCH / 4) {
+        xo[nxt][0] = xa[(s + 1) * 4 * TS], xo[nxt][1] = xa[(s + 1) * 4 * TS + 1];
+        yo[nxt][0] = ya[(s + 1) * 4 * TS], yo[nxt][1] = ya[(s + 1) * 4 * TS + 1];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      acc[0][0] = R::mfma(xo[cur][0], yo[cur][0], acc[0][0]);
+      acc[0][1] = R::mfma(xo[cur][0], yo[cur][1], acc[0][1]);
+      acc[1][0] = R::mfma(xo[cur][1], yo[cur][0], acc[1][0]);
+      acc[1][1] = R::mfma(xo[cur][1], yo[cur][1], acc[1][1]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
   long b0 = 0;
