@@ -86,11 +86,11 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  Renumbered so that one XCD
   // gets a contiguous run of tiles in column-major order: a few tile columns, i.e. a few hundred KB of
   // y plus all of x, instead of all of x and y per L2.
-  const long ntiles = a.tiles_i * a.tiles_j;
-  const long per_xcd = (ntiles + 7) / 8;
-  const long tile = (long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  const unsigned ntiles = (unsigned)(a.tiles_i * a.tiles_j);  // < 2^31, checked by the launcher
+  const unsigned per_xcd = (ntiles + 7) / 8;
+  const unsigned tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (tile >= ntiles) return;  // whole workgroup, before any barrier
-  const long jt = tile / a.tiles_i, it = tile % a.tiles_i;
+  const long jt = tile / (unsigned)a.tiles_i, it = tile % (unsigned)a.tiles_i;
   const long i0 = it * TS, j0 = jt * TS;
 
   // thread's share of the tile in row-major order: VW columns of PASSES rows
@@ -106,12 +106,30 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   // order below: first what the first MFMA needs (chunk 0 of x and y, mostly L2 hits), and the Cij
   // tile (HBM) only while the second-to-last chunk is being computed.
   T sx[SP][VW], sy[SP][VW];
+  // element offsets of this thread's vectors in chunk 0; chunk c is c * KCH rows further on
+  long xoff[SP], yoff[SP];
+#pragma unroll
+  for (int m = 0; m < SP; m++) {
+    xoff[m] = (long)(er + RPP * m) * a.N + i0 + VW * eg;
+    yoff[m] = (long)(er + RPP * m) * a.M + ecol;
+  }
+  const bool xcol_ok = i0 + VW * eg < a.N, ycol_ok = ecol < a.M;  // VEC: a vector is all in or all out
   auto request_chunk = [&](long b0) {
 #pragma unroll
     for (int m = 0; m < SP; m++) {
-      const long b = b0 + er + RPP * m;
-      load_vw_raw<T, VEC>(sx[m], a.x, b * a.N, i0 + VW * eg, a.N, b < a.B);
-      load_vw_raw<T, VEC>(sy[m], a.y, b * a.M, ecol, a.M, b < a.B);
+      const bool row_ok = b0 + er + RPP * m < a.B;
+      if (VEC) {
+        const typename R::vec_t vx =
+            *reinterpret_cast<const typename R::vec_t *>(a.x + ((row_ok && xcol_ok) ? xoff[m] + b0 * a.N : 0));
+        const typename R::vec_t vy =
+            *reinterpret_cast<const typename R::vec_t *>(a.y + ((row_ok && ycol_ok) ? yoff[m] + b0 * a.M : 0));
+#pragma unroll
+        for (int e = 0; e < VW; e++) sx[m][e] = vx[e], sy[m][e] = vy[e];
+      } else {
+        const long b = b0 + er + RPP * m;
+        load_vw_raw<T, false>(sx[m], a.x, b * a.N, i0 + VW * eg, a.N, row_ok);
+        load_vw_raw<T, false>(sy[m], a.y, b * a.M, ecol, a.M, row_ok);
+      }
     }
   };
   request_chunk(0);
@@ -161,16 +179,22 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
 
   // ---- chunks of the batch.  The loads of chunk c+1 are issued before chunk c is consumed from LDS,
   // so their latency hides behind the MFMA loop and the column sums.
+  const bool interior = i0 + TS <= a.N && j0 + TS <= a.M;  // the tile lies wholly inside the matrix
   auto chunk = [&](long b0, auto with_tile) {
     if (b0 > 0) {
       __syncthreads();  // previous chunk fully consumed
       SB_PHASE_MARK(2 * (int)(b0 / KCH));
     }
+    if (!(interior && b0 + KCH <= a.B)) {  // uniform: only edge tiles and a short last chunk zero-fill
+#pragma unroll
+      for (int m = 0; m < SP; m++) {
+        const long b = b0 + er + RPP * m;
+        zero_invalid<T, VEC>(sx[m], i0 + VW * eg, a.N, b < a.B);
+        zero_invalid<T, VEC>(sy[m], ecol, a.M, b < a.B);
+      }
+    }
 #pragma unroll
     for (int m = 0; m < SP; m++) {
-      const long b = b0 + er + RPP * m;
-      zero_invalid<T, VEC>(sx[m], i0 + VW * eg, a.N, b < a.B);
-      zero_invalid<T, VEC>(sy[m], ecol, a.M, b < a.B);
       typename R::vec_t vx, vy;
 #pragma unroll
       for (int e = 0; e < VW; e++) {
@@ -261,30 +285,37 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   __syncthreads();  // accumulator tile and reciprocals published
   SB_PHASE_MARK(13);
 
-  // ---- epilogue: decay + clamp, weight, mask, stores
+  // ---- epilogue: decay + clamp, weight, mask, stores.  Whether a synapse keeps its weight (row and
+  // column above the trace threshold, mask bit set) is combined into one predicate per element.
   const T scale = a.invB * a.tau;
   const bool masked = a.wmask != nullptr;
   T rcj[VW];
+  bool col_live[VW];
 #pragma unroll
-  for (int e = 0; e < VW; e++) rcj[e] = rcj_s[VW * eg + e];
+  for (int e = 0; e < VW; e++) {
+    rcj[e] = rcj_s[VW * eg + e];
+    col_live[e] = !(rcj[e] < T(0));
+  }
+  const long pass_stride = (long)RPP * a.M;
+  T *cij_row = a.Cij + (i0 + er) * a.M, *w_row = a.W + (i0 + er) * a.M;
 #pragma unroll
   for (int k = 0; k < PASSES; k++) {
     const int lr = er + RPP * k;
-    const long row = i0 + lr;
-    if (row >= a.N) continue;
+    if (i0 + lr >= a.N) continue;
     const T rci = rci_s[lr];
+    const bool row_live = !(rci < T(0)) && (MB != 1 || !masked || mb[k][0] != 0);
     T cv[VW], wv[VW];
 #pragma unroll
     for (int e = 0; e < VW; e++) {
       T cn = cpre[k][e] * a.omt + cs[lr * CP + VW * eg + e] * scale;
       cn = fmax(cn, T(0));  // 0 as well when cn is NaN, like the reference's `cn > 0 ? cn : 0`
       cv[e] = cn;
-      const T wgt = weight_from_traces<T>(cn, rci, rcj[e], a.cthr4);
-      const bool on = !masked || mb[k][MB == 1 ? 0 : e] != 0;
-      wv[e] = on ? wgt : T(0);
+      const T wgt = R::wlog(fmax(cn, a.cthr4) * rci * rcj[e]);
+      const bool keep = row_live && col_live[e] && (MB == 1 || !masked || mb[k][e] != 0);
+      wv[e] = keep ? wgt : T(0);
     }
-    store_vw<T, VEC>(cv, a.Cij + row * a.M, ecol, a.M);
-    store_vw<T, VEC>(wv, a.W + row * a.M, ecol, a.M);
+    store_vw<T, VEC>(cv, cij_row + k * pass_stride, ecol, a.M);
+    store_vw<T, VEC>(wv, w_row + k * pass_stride, ecol, a.M);
   }
   SB_PHASE_MARK(14);
 }
