@@ -40,10 +40,23 @@ struct ForwardArgs {
 // is loads + MFMAs + pointer bumps only.  The last, partial K chunk takes the guarded path.
 // One workgroup per CU is all the tiling provides at small batch sizes, so the register allocator is told
 // to aim for NWAVES/4 wavefronts per SIMD and spend the registers on loads in flight instead.
-template <typename T, int NG, bool FUSE, bool VEC, int NWAVES>
+//
+// LW: column blocks of the LAST group (1..VW).  A hypercolumn of 100 columns needs 7 blocks of 16, not
+// 8: with LW = 3 the last group's lanes load LW consecutive columns (12 bytes) instead of VW, and a
+// quarter of that group's MFMAs disappears.  The launcher picks LW < VW only when no vector of the last
+// group straddles the end of the tile.
+template <typename T, int LW>
+struct PackedCols {  // LW consecutive elements, element-aligned
+  T v[LW];
+} __attribute__((packed, aligned(sizeof(T))));
+
+template <typename T, int NG, bool FUSE, bool VEC, int NWAVES, int LW = Real<T>::VW>
 __global__ __launch_bounds__(64 * NWAVES) __attribute__((amdgpu_waves_per_eu(NWAVES / 4, NWAVES / 4)))
 void k_forward(ForwardArgs<T> a) {
   constexpr int VW = Real<T>::VW;
+  static_assert(LW >= 1 && LW <= VW, "width of the last group");
+  auto gwidth = [](int g) { return g == NG - 1 ? LW : VW; };         // column blocks of group g
+  auto gcol = [&](int g, int p_) { return g * (16 * VW) + gwidth(g) * p_; };  // first tile column of lane p_
   constexpr int GW = 16 * VW;
   constexpr int CP = NG * GW + VW;
   constexpr int KC = 4 * VW;  // k per chunk
@@ -83,7 +96,8 @@ void k_forward(ForwardArgs<T> a) {
 #pragma unroll
       for (int g = 0; g < NG; g++)
 #pragma unroll
-        for (int c = 0; c < VW; c++) acc[g][c] = Real<T>::mfma(xi[s], wi[s][g][c], acc[g][c]);
+        for (int c = 0; c < VW; c++)
+          if (c < gwidth(g)) acc[g][c] = Real<T>::mfma(xi[s], wi[s][g][c], acc[g][c]);
   };
   auto load_guarded = [&](long kc, T(&xo)[VW], T(&wo)[VW][NG][VW]) {
     const long kk = kc * KC + VW * q;
@@ -93,8 +107,17 @@ void k_forward(ForwardArgs<T> a) {
       const long krow = kk + s;
       const T *wrow = a.W + krow * a.M;
 #pragma unroll
-      for (int g = 0; g < NG; g++)
-        load_vw<T, VEC>(wo[s][g], wrow, j0 + g * GW + VW * p, jend, krow < a.N);
+      for (int g = 0; g < NG; g++) {
+        if (gwidth(g) == VW) {
+          load_vw<T, VEC>(wo[s][g], wrow, j0 + g * GW + VW * p, jend, krow < a.N);
+        } else {
+#pragma unroll
+          for (int e = 0; e < LW; e++) {
+            const long col = j0 + gcol(g, p) + e;
+            wo[s][g][e] = (krow < a.N && col < jend) ? wrow[col] : T(0);
+          }
+        }
+      }
     }
   };
 
@@ -109,7 +132,7 @@ void k_forward(ForwardArgs<T> a) {
     for (int s = 0; s < VW; s++)
 #pragma unroll
       for (int g = 0; g < NG; g++) {
-        long col = j0 + g * GW + VW * p;
+        long col = j0 + gcol(g, p);
         if (col >= jend) col = j0;  // redirected: feeds unused columns only
         wp[s][g] = a.W + ((long)w * KC + VW * q + s) * a.M + col;
       }
@@ -128,9 +151,15 @@ void k_forward(ForwardArgs<T> a) {
       for (int s = 0; s < VW; s++)
 #pragma unroll
         for (int g = 0; g < NG; g++) {
-          const vec_t wv = *reinterpret_cast<const vec_t *>(wp[s][g]);
+          if (gwidth(g) == VW) {
+            const vec_t wv = *reinterpret_cast<const vec_t *>(wp[s][g]);
 #pragma unroll
-          for (int e = 0; e < VW; e++) wo[s][g][e] = wv[e];
+            for (int e = 0; e < VW; e++) wo[s][g][e] = wv[e];
+          } else {
+            const PackedCols<T, LW> wv = *reinterpret_cast<const PackedCols<T, LW> *>(wp[s][g]);
+#pragma unroll
+            for (int e = 0; e < LW; e++) wo[s][g][e] = wv.v[e];
+          }
           wp[s][g] += advance ? wstep : 0;
         }
     };
@@ -179,10 +208,16 @@ void k_forward(ForwardArgs<T> a) {
     for (int g = 0; g < NG; g++)
 #pragma unroll
       for (int v = 0; v < 4; v++) {
-        vec_t t;
+        T *slot = &red[w - HALF][Real<T>::acc_row(q, v)][gcol(g, p)];
+        if (gwidth(g) == VW) {
+          vec_t t;
 #pragma unroll
-        for (int c = 0; c < VW; c++) t[c] = acc[g][c][v];
-        *reinterpret_cast<vec_t *>(&red[w - HALF][Real<T>::acc_row(q, v)][g * GW + VW * p]) = t;
+          for (int c = 0; c < VW; c++) t[c] = acc[g][c][v];
+          *reinterpret_cast<vec_t *>(slot) = t;
+        } else {
+#pragma unroll
+          for (int c = 0; c < LW; c++) slot[c] = acc[g][c][v];
+        }
       }
   }
   __syncthreads();
@@ -191,11 +226,16 @@ void k_forward(ForwardArgs<T> a) {
     for (int g = 0; g < NG; g++)
 #pragma unroll
       for (int v = 0; v < 4; v++) {
-        vec_t *slot = reinterpret_cast<vec_t *>(&red[w][Real<T>::acc_row(q, v)][g * GW + VW * p]);
-        vec_t t = *slot;
+        T *slot = &red[w][Real<T>::acc_row(q, v)][gcol(g, p)];
+        if (gwidth(g) == VW) {
+          vec_t t = *reinterpret_cast<vec_t *>(slot);
 #pragma unroll
-        for (int c = 0; c < VW; c++) t[c] += acc[g][c][v];
-        *slot = t;
+          for (int c = 0; c < VW; c++) t[c] += acc[g][c][v];
+          *reinterpret_cast<vec_t *>(slot) = t;
+        } else {
+#pragma unroll
+          for (int c = 0; c < LW; c++) slot[c] += acc[g][c][v];
+        }
       }
   }
   __syncthreads();

@@ -61,6 +61,21 @@ int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias
   if (softmax && need <= max_fused) {
     const bool vec = base_vec && (Mc % VW == 0);
     a.col_tiles = H;
+    // Hypercolumns that need 7 column blocks of 16 (97..112 columns, e.g. 100): the last group runs
+    // with 3 (float) or 1 (double) blocks instead of VW, provided none of its vectors straddles the
+    // end of the hypercolumn.
+    const long nblocks = cdiv(Mc, 16);
+    if (vec && nblocks == 7) {
+      constexpr int NGL = 8 / VW, LWL = 7 - (NGL - 1) * VW;  // float: 2 groups, 3 blocks; double: 4, 1
+      if ((Mc - (NGL - 1) * GW) % LWL == 0) {
+        ProfScope prof_(st, K_FORWARD);
+        const long grid = 8 * cdiv(a.col_tiles * a.batch_tiles, 8);
+        SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
+        hipLaunchKernelGGL((k_forward<T, NGL, true, true, 8, LWL>), dim3((unsigned)grid), dim3(512), 0, st, a);
+        SB_LAUNCH_CHECK();
+        return 0;
+      }
+    }
     if (need <= 1) return forward_variant<T, 1, true>(st, a, vec);
     if (need <= 2) return forward_variant<T, 2, true>(st, a, vec);
     if (need <= 4) return forward_variant<T, 4, true>(st, a, vec);
