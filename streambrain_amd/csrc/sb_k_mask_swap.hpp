@@ -76,6 +76,253 @@ __device__ __forceinline__ RowCand<T> pick_first(RowCand<T> a, RowCand<T> b) {
   return take ? b : a;
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Fast path of the swap loop.  Over at most 16 iterations only the 16 best silent rows and the 16 worst
+// active rows of the INITIAL state (plus rows that changed sides on the way) can ever be picked, because
+// an iteration changes nothing but the two rows it swaps.  So:
+//   phase A (whole workgroup): a radix select on monotone integer keys of the scores finds a threshold
+//     per group such that the rows beyond it are a small superset of those 16; a large group of exactly
+//     equal scores at the threshold (rows of dead inputs all score 0) is cut down to its highest indices,
+//     which is the order the tie rule would take them in;
+//   phase B (one wavefront, one candidate per lane and group): the iterations themselves, with the same
+//     picks, tie rule, break conditions and score expression as the full scan.
+// Anything the fast path does not cover (NaN scores, more iterations, too many near-equal candidates)
+// returns false and the caller runs the full scan.
+template <typename T>
+struct ScoreKey;
+template <>
+struct ScoreKey<float> {
+  using K = uint32_t;
+  static constexpr int BITS = 32, PASSES = 2;
+  static __device__ __forceinline__ K of(float s) {
+    const uint32_t b = __float_as_uint(s + 0.0f);  // -0 and +0 compare equal, so they share a key
+    return b ^ ((b >> 31) ? 0xffffffffu : 0x80000000u);
+  }
+};
+template <>
+struct ScoreKey<double> {
+  using K = uint64_t;
+  static constexpr int BITS = 64, PASSES = 3;
+  static __device__ __forceinline__ K of(double s) {
+    const uint64_t b = (uint64_t)__double_as_longlong(s + 0.0);
+    return b ^ ((b >> 63) ? ~0ull : (1ull << 63));
+  }
+};
+__device__ __forceinline__ float readlane_t(float v, int l) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l));
+}
+__device__ __forceinline__ double readlane_t(double v, int l) {
+  const long long b = __double_as_longlong(v);
+  const int lo = __builtin_amdgcn_readlane((int)(b & 0xffffffffLL), l);
+  const int hi = __builtin_amdgcn_readlane((int)(b >> 32), l);
+  return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+
+template <typename T, int NT, int R>
+struct MaskSwapFast {
+  using SK = ScoreKey<T>;
+  using K = typename SK::K;
+  static constexpr int TOPK = 16, CAP = 48, DIG = 11, BINS = 1 << DIG, PER = BINS / NT, NWV = NT / 64;
+  static constexpr int ISH = NT * R > BINS ? 2 : 0;  // index bins of the tie cut: (row index) >> ISH
+  static_assert(NT * R <= (BINS << 2) && BINS % NT == 0, "row indices must fit the index histogram");
+  struct Shared {
+    unsigned hist[2][BINS];
+    int cand[2][64];
+    int ncand[2], sel_bin[2], sel_above[2], wtot[2][NWV];
+    K eq_min[2], eq_max[2];
+  };
+
+  // Largest bin b with (rows in bins >= b) >= need, per group; sel_bin stays -1 when the histogram holds
+  // fewer than `need` rows.  Two barriers inside.
+  static __device__ void crossing(Shared &sh, const int (&need)[2], const bool (&active)[2]) {
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    int c[2], incl[2];
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+      c[g] = 0;
+#pragma unroll
+      for (int b = 0; b < PER; b++) c[g] += (int)sh.hist[g][PER * tid + b];
+      int s = c[g];
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {  // inclusive suffix sum inside the wavefront
+        const int v = __shfl_down(s, o);
+        if (lane + o < 64) s += v;
+      }
+      incl[g] = s;
+      if (lane == 0) sh.wtot[g][wv] = s;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+      for (int w2 = wv + 1; w2 < NWV; w2++) incl[g] += sh.wtot[g][w2];
+      const int after = incl[g] - c[g];
+      if (active[g] && after < need[g] && need[g] <= incl[g]) {  // exactly one thread per group
+        int acc = after;
+        for (int b = PER - 1; b >= 0; b--) {
+          const int hb = (int)sh.hist[g][PER * tid + b];
+          if (acc + hb >= need[g]) {
+            sh.sel_bin[g] = PER * tid + b;
+            sh.sel_above[g] = acc;
+            break;
+          }
+          acc += hb;
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+  static __device__ void clear(Shared &sh) {
+    for (int i = threadIdx.x; i < 2 * BINS; i += NT) (&sh.hist[0][0])[i] = 0u;
+    if (threadIdx.x < 2) sh.sel_bin[threadIdx.x] = -1;
+  }
+
+  // true: the swaps are done and written back; false: nothing was changed, run the full scan
+  static __device__ bool run(const MaskArgs<T> &a, Shared &sh, const T (&score)[R], const int (&m)[R]) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    K key[R];
+#pragma unroll
+    for (int k = 0; k < R; k++) {
+      const K u = SK::of(score[k]);
+      key[k] = m[k] == 0 ? u : (K)~u;  // in both groups the wanted rows are those with the LARGEST keys
+    }
+    K prefix[2] = {0, 0};
+    int need[2] = {TOPK, TOPK};
+    bool all[2] = {false, false};  // the whole group is wanted (it has fewer than TOPK rows)
+    // ---- phase A: threshold on the leading DIG * PASSES key bits
+#pragma unroll
+    for (int p = 0; p < SK::PASSES; p++) {
+      const int shift = SK::BITS - DIG * (p + 1);
+      clear(sh);
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < R; k++) {
+        const int g = m[k];
+        if (g < 2 && !all[g] && (p == 0 || (key[k] >> (shift + DIG)) == prefix[g]))
+          atomicAdd(&sh.hist[g][(unsigned)(key[k] >> shift) & (BINS - 1)], 1u);
+      }
+      __syncthreads();
+      const bool active[2] = {!all[0], !all[1]};
+      crossing(sh, need, active);
+#pragma unroll
+      for (int g = 0; g < 2; g++) {
+        if (all[g]) continue;
+        if (sh.sel_bin[g] < 0) {
+          all[g] = true;
+        } else {
+          prefix[g] = (prefix[g] << DIG) | (K)sh.sel_bin[g];
+          need[g] -= sh.sel_above[g];
+        }
+      }
+      __syncthreads();  // everybody has read the selection before the next pass clears it
+    }
+    constexpr int TAIL = SK::BITS - DIG * SK::PASSES;  // key bits below the threshold's resolution
+    // ---- candidates: rows at or beyond the threshold
+    if (tid < 2) {
+      sh.ncand[tid] = 0;
+      sh.eq_min[tid] = ~(K)0;
+      sh.eq_max[tid] = 0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < R; k++) {
+      const int g = m[k];
+      if (g >= 2) continue;
+      const K top = key[k] >> TAIL;
+      if (all[g] || top >= prefix[g]) {
+        const int pos = atomicAdd(&sh.ncand[g], 1);
+        if (pos < 64) sh.cand[g][pos] = tid + NT * k;
+      }
+      if (!all[g] && top == prefix[g]) {
+        atomicMin(&sh.eq_min[g], key[k]);
+        atomicMax(&sh.eq_max[g], key[k]);
+      }
+    }
+    __syncthreads();
+    // ---- too many candidates: a block of exactly equal scores at the threshold is cut down to its
+    // `need` highest row indices (the tie rule takes equal scores from the highest index down)
+    bool cut[2];
+    bool any_cut = false;
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+      cut[g] = sh.ncand[g] > CAP;
+      if (cut[g] && sh.eq_min[g] != sh.eq_max[g]) return false;  // uniform: read from LDS by everybody
+      any_cut |= cut[g];
+    }
+    if (any_cut) {
+      __syncthreads();
+      clear(sh);
+      if (tid < 2 && cut[tid]) sh.ncand[tid] = 0;
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < R; k++) {
+        const int g = m[k];
+        if (g < 2 && cut[g] && (key[k] >> TAIL) == prefix[g]) atomicAdd(&sh.hist[g][(tid + NT * k) >> ISH], 1u);
+      }
+      __syncthreads();
+      crossing(sh, need, cut);
+#pragma unroll
+      for (int k = 0; k < R; k++) {
+        const int g = m[k];
+        if (g >= 2 || !cut[g]) continue;
+        const K top = key[k] >> TAIL;
+        const int i = tid + NT * k;
+        if (top > prefix[g] || (top == prefix[g] && (i >> ISH) >= sh.sel_bin[g])) {
+          const int pos = atomicAdd(&sh.ncand[g], 1);
+          if (pos < 64) sh.cand[g][pos] = i;
+        }
+      }
+      __syncthreads();
+      if (sh.ncand[0] > CAP || sh.ncand[1] > CAP) return false;
+    }
+    if (tid >= 64) return true;  // phase B is the first wavefront's
+
+    // ---- phase B: lane l holds silent candidate l and active candidate l
+    int nS = sh.ncand[0], nA = sh.ncand[1];
+    bool vS = lane < nS, vA = lane < nA;
+    int iS = vS ? sh.cand[0][lane] : 0, iA = vA ? sh.cand[1][lane] : 0;
+    T nomS = a.nom[iS], nomA = a.nom[iA];
+    int csS = a.csum[iS], csA = a.csum[iA];
+    T scS = mask_score<T>(nomS, csS), scA = mask_score<T>(nomA, csA);
+    for (long it = 0; it < a.iterations; it++) {
+      RowCand<T> cmax{scS, vS ? iS : -1}, cmin{scA, vA ? iA : -1};
+      SB_ROW_REDUCE(pick_max<T>, cmax);
+      SB_ROW_REDUCE(pick_min<T>, cmin);
+#pragma unroll
+      for (int o = 16; o <= 32; o <<= 1) {
+        cmax = pick_max<T>(cmax, shfl_xor_cand<T>(cmax, o));
+        cmin = pick_min<T>(cmin, shfl_xor_cand<T>(cmin, o));
+      }
+      if (cmax.idx < 0 || cmin.idx < 0) break;  // no silent or no active row
+      if (cmax.val < cmin.val) break;
+      const int lS = __builtin_ctzll(__ballot(vS && iS == cmax.idx));
+      const int lA = __builtin_ctzll(__ballot(vA && iA == cmin.idx));
+      const T nomW = readlane_t(nomS, lS), nomL = readlane_t(nomA, lA);
+      const int csW = __builtin_amdgcn_readlane(csS, lS), csL = __builtin_amdgcn_readlane(csA, lA);
+      if (lane == lS) vS = false;
+      if (lane == lA) vA = false;
+      if (lane == nA) {  // the best silent row becomes active
+        vA = true, iA = cmax.idx, nomA = nomW, csA = csW + 1;
+        scA = mask_score<T>(nomA, csA);
+      }
+      if (lane == nS) {  // the worst active row becomes silent
+        vS = true, iS = cmin.idx, nomS = nomL, csS = csL - 1;
+        scS = mask_score<T>(nomS, csS);
+      }
+      nA++, nS++;
+    }
+    if (vS) {
+      a.wmask[(long)iS * a.H + a.h] = 0;
+      a.csum[iS] = csS;
+    }
+    if (vA) {
+      a.wmask[(long)iA * a.H + a.h] = 1;
+      a.csum[iA] = csA;
+    }
+    return true;
+  }
+};
+
 // NT threads (a multiple of 64, at most 256: one wavefront per SIMD, so the replicated reduction code
 // is not time-shared), thread t owns rows t, t+NT, ..., t+(R-1)*NT.
 template <typename T, int NT, int R>
@@ -108,6 +355,11 @@ __global__ __launch_bounds__(NT) void k_mask_swap_reg(MaskArgs<T> a) {
   // NaN scores need the "first candidate" bookkeeping of the sequential scan; without any NaN (the
   // normal case; a score is NaN iff its nominator is) that half of the reduction is skipped
   const bool track_first = __syncthreads_or(has_nan) != 0;
+  if (!track_first && a.iterations <= MaskSwapFast<T, NT, R>::TOPK) {
+    __shared__ typename MaskSwapFast<T, NT, R>::Shared fast_lds;
+    if (MaskSwapFast<T, NT, R>::run(a, fast_lds, score, m)) return;
+    __syncthreads();
+  }
 
   for (long it = 0; it < a.iterations; it++) {
     const int buf = (int)(it & 1);

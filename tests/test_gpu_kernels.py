@@ -177,6 +177,42 @@ def test_update_mask_ties_and_degenerate_columns(k, oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("N,H,Mc", [(1568, 30, 100), (300, 4, 10), (6000, 3, 8)])
+@pytest.mark.parametrize("kind", ["dead_rows", "near_equal", "identical_rows", "few_active", "few_silent"])
+def test_update_mask_tie_blocks(k, oracle, dtype, N, H, Mc, kind):
+    """Score distributions that stress the candidate preselection of the swap loop: large blocks of
+    exactly equal scores (dead inputs score 0), many nearly equal scores, tiny groups."""
+    rng = np.random.default_rng(N + len(kind))
+    wmask, W, Ci, Cj, Cij = _mask_problem(rng, N, H, Mc, dtype, density=0.3)
+    h = 1
+    if kind == "dead_rows":
+        dead = rng.random(N) < 0.6
+        Ci[dead] = 0.001  # below cthr: nominator 0, score 0 whatever csum is
+    elif kind == "near_equal":
+        Ci[:] = 0.4
+        # distinct scores, 2e-6 apart (relative): far above rounding noise, far below the preselection's
+        # resolution, so dozens of rows share the threshold bucket
+        Cij[:] = (Cij[0:1, :] * (1 + 2e-6 * rng.permutation(N)[:, None])).astype(dtype)
+        W[:] = W[0:1, :]
+    elif kind == "identical_rows":
+        Ci[:] = 0.4
+        Cij[:] = Cij[0:1, :]
+        W[:] = W[0:1, :]
+        wmask[:] = 0
+        wmask[rng.random(N) < 0.3, h] = 1  # equal csum inside each group: all scores of a group tie
+    elif kind == "few_active":
+        wmask[:, h] = 0
+        wmask[rng.choice(N, 5, replace=False), h] = 1
+    elif kind == "few_silent":
+        wmask[:, h] = 1
+        wmask[rng.choice(N, 7, replace=False), h] = 0
+    trace = {}
+    ref = oracle.update_mask(wmask.copy(), W, Ci, Cj, Cij, 0.01, H, Mc, h, 16, trace=trace)
+    got = k.update_mask(wmask.copy(), W, Ci, Cj, Cij, 0.01, H, Mc, h, 16)
+    assert np.array_equal(got, ref), f"masks differ in {(got != ref).sum()} entries, swaps {trace['swaps']}"
+
+
+@pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("N", [24, 700, 3000])
 def test_update_mask_nan_scores(k, oracle, dtype, N):
     """Rows with Ci = 1 and Cij = Cj give 0 * log(x/0) = NaN nominators.  The reference's sequential
