@@ -118,6 +118,47 @@ __device__ __forceinline__ double readlane_t(double v, int l) {
   return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
 }
 
+// (key, row index) pairs and their wavefront-wide maximum; idx < 0 marks "no candidate"
+template <typename K>
+struct KeyIdx {
+  K key;
+  int idx;
+};
+template <typename K>
+__device__ __forceinline__ KeyIdx<K> pick_key(KeyIdx<K> a, KeyIdx<K> b) {
+  const bool take = b.idx >= 0 && (a.idx < 0 || b.key > a.key || (b.key == a.key && b.idx > a.idx));
+  return take ? b : a;
+}
+__device__ __forceinline__ uint32_t readlane_k(uint32_t v, int l) {
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, l);
+}
+__device__ __forceinline__ uint64_t readlane_k(uint64_t v, int l) {
+  const uint32_t lo = readlane_k((uint32_t)v, l), hi = readlane_k((uint32_t)(v >> 32), l);
+  return ((uint64_t)hi << 32) | lo;
+}
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_move_k(uint32_t v) {
+  return (uint32_t)dpp_move<CTRL>((int)v);
+}
+template <int CTRL>
+__device__ __forceinline__ uint64_t dpp_move_k(uint64_t v) {
+  return ((uint64_t)dpp_move_k<CTRL>((uint32_t)(v >> 32)) << 32) | dpp_move_k<CTRL>((uint32_t)v);
+}
+template <typename K, int CTRL>
+__device__ __forceinline__ KeyIdx<K> dpp_keyidx(KeyIdx<K> c) {
+  return KeyIdx<K>{dpp_move_k<CTRL>(c.key), dpp_move<CTRL>(c.idx)};
+}
+template <typename K>
+__device__ __forceinline__ KeyIdx<K> wave_pick(KeyIdx<K> c) {  // every lane ends with the result
+  c = pick_key<K>(c, dpp_keyidx<K, kDppSwap1>(c));
+  c = pick_key<K>(c, dpp_keyidx<K, kDppSwap2>(c));
+  c = pick_key<K>(c, dpp_keyidx<K, kDppHalfMirror>(c));
+  c = pick_key<K>(c, dpp_keyidx<K, kDppMirror>(c));
+#pragma unroll
+  for (int o = 16; o <= 32; o <<= 1) c = pick_key<K>(c, KeyIdx<K>{(K)__shfl_xor(c.key, o), __shfl_xor(c.idx, o)});
+  return c;
+}
+
 template <typename T, int NT, int R>
 struct MaskSwapFast {
   using SK = ScoreKey<T>;
@@ -277,37 +318,38 @@ struct MaskSwapFast {
     }
     if (tid >= 64) return true;  // phase B is the first wavefront's
 
-    // ---- phase B: lane l holds silent candidate l and active candidate l
+    // ---- phase B: lane l holds silent candidate l and active candidate l.  A pick is the maximum of
+    // (key, row index) pairs -- the key orders the scores, the index settles equal scores in favour of
+    // the later row, as the sequential >= / <= scans do.  A row that changes sides takes the score of
+    // its other side along (csum +- 1), computed once up front, so the loop holds no division.
     int nS = sh.ncand[0], nA = sh.ncand[1];
     bool vS = lane < nS, vA = lane < nA;
     int iS = vS ? sh.cand[0][lane] : 0, iA = vA ? sh.cand[1][lane] : 0;
-    T nomS = a.nom[iS], nomA = a.nom[iA];
     int csS = a.csum[iS], csA = a.csum[iA];
-    T scS = mask_score<T>(nomS, csS), scA = mask_score<T>(nomA, csA);
+    const T nomS = a.nom[iS], nomA = a.nom[iA];
+    // keys as seen from the silent side (largest score wins) and from the active side (smallest wins)
+    K kS = SK::of(mask_score<T>(nomS, csS)), kS_other = (K)~SK::of(mask_score<T>(nomS, csS + 1));
+    K kA = (K)~SK::of(mask_score<T>(nomA, csA)), kA_other = SK::of(mask_score<T>(nomA, csA - 1));
     for (long it = 0; it < a.iterations; it++) {
-      RowCand<T> cmax{scS, vS ? iS : -1}, cmin{scA, vA ? iA : -1};
-      SB_ROW_REDUCE(pick_max<T>, cmax);
-      SB_ROW_REDUCE(pick_min<T>, cmin);
-#pragma unroll
-      for (int o = 16; o <= 32; o <<= 1) {
-        cmax = pick_max<T>(cmax, shfl_xor_cand<T>(cmax, o));
-        cmin = pick_min<T>(cmin, shfl_xor_cand<T>(cmin, o));
-      }
+      KeyIdx<K> cmax{kS, vS ? iS : -1}, cmin{kA, vA ? iA : -1};
+      cmax = wave_pick<K>(cmax);
+      cmin = wave_pick<K>(cmin);
       if (cmax.idx < 0 || cmin.idx < 0) break;  // no silent or no active row
-      if (cmax.val < cmin.val) break;
+      if (cmax.key < (K)~cmin.key) break;       // vmax0 < vmin1
       const int lS = __builtin_ctzll(__ballot(vS && iS == cmax.idx));
       const int lA = __builtin_ctzll(__ballot(vA && iA == cmin.idx));
-      const T nomW = readlane_t(nomS, lS), nomL = readlane_t(nomA, lA);
+      const K wOther = readlane_k(kS_other, lS), wThis = cmax.key;  // winner: its active-side key, ...
+      const K lOther = readlane_k(kA_other, lA), lThis = cmin.key;
       const int csW = __builtin_amdgcn_readlane(csS, lS), csL = __builtin_amdgcn_readlane(csA, lA);
       if (lane == lS) vS = false;
       if (lane == lA) vA = false;
       if (lane == nA) {  // the best silent row becomes active
-        vA = true, iA = cmax.idx, nomA = nomW, csA = csW + 1;
-        scA = mask_score<T>(nomA, csA);
+        vA = true, iA = cmax.idx, csA = csW + 1;
+        kA = wOther, kA_other = wThis;
       }
       if (lane == nS) {  // the worst active row becomes silent
-        vS = true, iS = cmin.idx, nomS = nomL, csS = csL - 1;
-        scS = mask_score<T>(nomS, csS);
+        vS = true, iS = cmin.idx, csS = csL - 1;
+        kS = lOther, kS_other = lThis;
       }
       nA++, nS++;
     }
