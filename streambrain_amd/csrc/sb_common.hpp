@@ -155,6 +155,71 @@ __device__ __forceinline__ void zero_invalid(T (&v)[Real<T>::VW], long col, long
   }
 }
 
+// A bounds-checked window of at most 2 GiB onto a global array, addressed through a buffer descriptor
+// with 32-bit byte offsets: a per-lane offset plus a wavefront-uniform one that lives in a scalar
+// register.  Accesses past the end of the window read zero and store nothing, in hardware; so a loop
+// over rows needs neither clamped addresses nor zero-filling nor branches, and advancing to the next
+// rows costs no vector instruction.  A lane whose vector lies outside the array in a way the window's
+// end does not express (a column beyond the row length) passes kOutside as its offset.
+template <typename T>
+struct BufferWindow {
+  static constexpr unsigned kOutside = 0x80000000u;  // beyond any window, also after adding a uniform offset
+  __amdgpu_buffer_rsrc_t rsrc;
+  __device__ BufferWindow(const T *base, long elems) {
+    const long bytes = elems * (long)sizeof(T);
+    // descriptor word 3 = 0x00020000: raw buffer, 32-bit data format, as for every untyped gfx9 buffer
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(base), 0,
+                                             (int)(bytes < 0x80000000L ? bytes : 0x80000000L), 0x00020000);
+  }
+  using u4 = unsigned __attribute__((ext_vector_type(4)));
+  using u2 = unsigned __attribute__((ext_vector_type(2)));
+  // `at`: byte offset of the vector's first element (ignored parts: see `col`, `limit`); VEC moves the
+  // VW elements as one 16-byte access (all inside or all outside), otherwise element by element with
+  // elements at columns >= limit excluded.
+  template <bool VEC>
+  __device__ __forceinline__ void load(T (&out)[Real<T>::VW], unsigned at, unsigned uniform, long col,
+                                       long limit) const {
+    constexpr int VW = Real<T>::VW;
+    if (VEC) {
+      const u4 raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(col < limit ? at : kOutside),
+                                                           (int)uniform, 0);
+      const typename Real<T>::vec_t v = __builtin_bit_cast(typename Real<T>::vec_t, raw);
+#pragma unroll
+      for (int e = 0; e < VW; e++) out[e] = v[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < VW; e++) {
+        const int o = (int)(col + e < limit ? at + e * (unsigned)sizeof(T) : kOutside);
+        if constexpr (sizeof(T) == 4)
+          out[e] = __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(rsrc, o, (int)uniform, 0));
+        else
+          out[e] = __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(rsrc, o, (int)uniform, 0));
+      }
+    }
+  }
+  template <bool VEC>
+  __device__ __forceinline__ void store(const T (&in)[Real<T>::VW], unsigned at, unsigned uniform, long col,
+                                        long limit) const {
+    constexpr int VW = Real<T>::VW;
+    if (VEC) {
+      typename Real<T>::vec_t v;
+#pragma unroll
+      for (int e = 0; e < VW; e++) v[e] = in[e];
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), rsrc,
+                                             (int)(col < limit ? at : kOutside), (int)uniform, 0);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VW; e++) {
+        const int o = (int)(col + e < limit ? at + e * (unsigned)sizeof(T) : kOutside);
+        if constexpr (sizeof(T) == 4)
+          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, in[e]), rsrc, o, (int)uniform, 0);
+        else
+          __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u2, in[e]), rsrc, o, (int)uniform, 0);
+      }
+    }
+  }
+};
+
 // Width-generic variants: W consecutive elements (W = 1, 2, 4 for float; 1, 2 for double), moved as one
 // W*sizeof(T)-byte access when VEC promises that alignment and limit % W == 0.
 template <typename T, int W>

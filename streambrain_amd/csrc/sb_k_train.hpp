@@ -101,35 +101,29 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   for (int z = 0; z < (int)(blockIdx.x / 256) * SB_STAGGER; z++) __builtin_amdgcn_s_sleep(16);
 #endif
   SB_PHASE_MARK(0);
-  // All global loads are branch-free (clamped addresses; what a guard excludes is zeroed or ignored
-  // where it is consumed), so they stay in flight together.  Loads return in issue order, hence the
-  // order below: first what the first MFMA needs (chunk 0 of x and y, mostly L2 hits), and the Cij
-  // tile (HBM) only while the second-to-last chunk is being computed.
+  // x, y, the Cij tile and the W tile are reached through bounds-checked buffer windows: rows past the
+  // batch or past the matrix read zero / store nothing in hardware, so there are no clamped addresses,
+  // no zero-filling and no branches, and the row advance per chunk / pass is a scalar offset.  Loads
+  // return in issue order, hence the order below: first what the first MFMA needs (chunk 0 of x and
+  // y, mostly L2 hits), and the Cij tile (HBM) only while the second-to-last chunk is being computed.
+  constexpr unsigned ES = sizeof(T);
+  const BufferWindow<T> xwin(a.x, a.B * a.N), ywin(a.y, a.B * a.M);
+  const long tile_rows = a.N - i0 < TS ? a.N - i0 : TS;
+  const BufferWindow<T> cwin(a.Cij + i0 * a.M, tile_rows * a.M), wwin(a.W + i0 * a.M, tile_rows * a.M);
   T sx[SP][VW], sy[SP][VW];
-  // element offsets of this thread's vectors in chunk 0; chunk c is c * KCH rows further on
-  long xoff[SP], yoff[SP];
+  // byte offsets of this thread's vectors in chunk 0; chunk c is c * KCH rows further on
+  unsigned xat[SP], yat[SP];
 #pragma unroll
   for (int m = 0; m < SP; m++) {
-    xoff[m] = (long)(er + RPP * m) * a.N + i0 + VW * eg;
-    yoff[m] = (long)(er + RPP * m) * a.M + ecol;
+    xat[m] = (unsigned)(((long)(er + RPP * m) * a.N + i0 + VW * eg) * ES);
+    yat[m] = (unsigned)(((long)(er + RPP * m) * a.M + ecol) * ES);
   }
-  const bool xcol_ok = i0 + VW * eg < a.N, ycol_ok = ecol < a.M;  // VEC: a vector is all in or all out
   auto request_chunk = [&](long b0) {
+    const unsigned xrow = (unsigned)(b0 * a.N * ES), yrow = (unsigned)(b0 * a.M * ES);
 #pragma unroll
     for (int m = 0; m < SP; m++) {
-      const bool row_ok = b0 + er + RPP * m < a.B;
-      if (VEC) {
-        const typename R::vec_t vx =
-            *reinterpret_cast<const typename R::vec_t *>(a.x + ((row_ok && xcol_ok) ? xoff[m] + b0 * a.N : 0));
-        const typename R::vec_t vy =
-            *reinterpret_cast<const typename R::vec_t *>(a.y + ((row_ok && ycol_ok) ? yoff[m] + b0 * a.M : 0));
-#pragma unroll
-        for (int e = 0; e < VW; e++) sx[m][e] = vx[e], sy[m][e] = vy[e];
-      } else {
-        const long b = b0 + er + RPP * m;
-        load_vw_raw<T, false>(sx[m], a.x, b * a.N, i0 + VW * eg, a.N, row_ok);
-        load_vw_raw<T, false>(sy[m], a.y, b * a.M, ecol, a.M, row_ok);
-      }
+      xwin.template load<VEC>(sx[m], xat[m], xrow, i0 + VW * eg, a.N);
+      ywin.template load<VEC>(sy[m], yat[m], yrow, ecol, a.M);
     }
   };
   request_chunk(0);
@@ -162,12 +156,11 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   }
 
   T cpre[PASSES][VW];  // Cij tile: VW columns of PASSES rows per thread
+  const unsigned tat = (unsigned)(((long)er * a.M + ecol) * ES);  // this thread's vector in pass 0
+  const unsigned pass_bytes = (unsigned)((long)RPP * a.M * ES);    // the next pass is RPP rows further on
   auto request_tile = [&]() {
 #pragma unroll
-    for (int k = 0; k < PASSES; k++) {
-      const long row = i0 + er + RPP * k;
-      load_vw_raw<T, VEC>(cpre[k], a.Cij, row * a.M, ecol, a.M, row < a.N);  // excluded parts are never stored
-    }
+    for (int k = 0; k < PASSES; k++) cwin.template load<VEC>(cpre[k], tat, k * pass_bytes, ecol, a.M);
   };
 
   acc_t acc[2][2];
@@ -179,19 +172,10 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
 
   // ---- chunks of the batch.  The loads of chunk c+1 are issued before chunk c is consumed from LDS,
   // so their latency hides behind the MFMA loop and the column sums.
-  const bool interior = i0 + TS <= a.N && j0 + TS <= a.M;  // the tile lies wholly inside the matrix
   auto chunk = [&](long b0, auto with_tile) {
     if (b0 > 0) {
       __syncthreads();  // previous chunk fully consumed
       SB_PHASE_MARK(2 * (int)(b0 / KCH));
-    }
-    if (!(interior && b0 + KCH <= a.B)) {  // uniform: only edge tiles and a short last chunk zero-fill
-#pragma unroll
-      for (int m = 0; m < SP; m++) {
-        const long b = b0 + er + RPP * m;
-        zero_invalid<T, VEC>(sx[m], i0 + VW * eg, a.N, b < a.B);
-        zero_invalid<T, VEC>(sy[m], ecol, a.M, b < a.B);
-      }
     }
 #pragma unroll
     for (int m = 0; m < SP; m++) {
@@ -206,7 +190,7 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
     }
     __syncthreads();
     SB_PHASE_MARK(1 + 2 * (int)(b0 / KCH));
-    request_chunk(b0 + KCH);  // past the batch: clamped loads nobody consumes
+    request_chunk(b0 + KCH);  // past the batch: reads zeros nobody consumes
     if (decltype(with_tile)::value) request_tile();
 
     if (summer) {
@@ -296,12 +280,9 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
     rcj[e] = rcj_s[VW * eg + e];
     col_live[e] = !(rcj[e] < T(0));
   }
-  const long pass_stride = (long)RPP * a.M;
-  T *cij_row = a.Cij + (i0 + er) * a.M, *w_row = a.W + (i0 + er) * a.M;
 #pragma unroll
   for (int k = 0; k < PASSES; k++) {
-    const int lr = er + RPP * k;
-    if (i0 + lr >= a.N) continue;
+    const int lr = er + RPP * k;  // rows past the matrix compute garbage that the window drops
     const T rci = rci_s[lr];
     const bool row_live = !(rci < T(0)) && (MB != 1 || !masked || mb[k][0] != 0);
     T cv[VW], wv[VW];
@@ -314,8 +295,8 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
       const bool keep = row_live && col_live[e] && (MB == 1 || !masked || mb[k][e] != 0);
       wv[e] = keep ? wgt : T(0);
     }
-    store_vw<T, VEC>(cv, cij_row + k * pass_stride, ecol, a.M);
-    store_vw<T, VEC>(wv, w_row + k * pass_stride, ecol, a.M);
+    cwin.template store<VEC>(cv, tat, k * pass_bytes, ecol, a.M);
+    wwin.template store<VEC>(wv, tat, k * pass_bytes, ecol, a.M);
   }
   SB_PHASE_MARK(14);
 }
