@@ -166,7 +166,7 @@ struct BufferWindow {
   static constexpr unsigned kOutside = 0x80000000u;  // beyond any window, also after adding a uniform offset
   __amdgpu_buffer_rsrc_t rsrc;
   __device__ BufferWindow(const T *base, long elems) {
-    const long bytes = elems * (long)sizeof(T);
+    const long bytes = elems > 0 ? elems * (long)sizeof(T) : 0;
     // descriptor word 3 = 0x00020000: raw buffer, 32-bit data format, as for every untyped gfx9 buffer
     rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(base), 0,
                                              (int)(bytes < 0x80000000L ? bytes : 0x80000000L), 0x00020000);
@@ -196,6 +196,27 @@ struct BufferWindow {
           out[e] = __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(rsrc, o, (int)uniform, 0));
       }
     }
+  }
+  // NE consecutive elements (4, 8, 12 or 16 bytes) as one access; element-aligned
+  template <int NE>
+  __device__ __forceinline__ void load_n(T (&out)[NE], unsigned at) const {
+    constexpr int BYTES = NE * (int)sizeof(T);
+    static_assert(BYTES == 4 || BYTES == 8 || BYTES == 12 || BYTES == 16, "one buffer access");
+    using u3 = unsigned __attribute__((ext_vector_type(3)));
+    unsigned raw[BYTES / 4];
+    if constexpr (BYTES == 4) {
+      raw[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)at, 0, 0);
+    } else if constexpr (BYTES == 8) {
+      const u2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)at, 0, 0);
+      raw[0] = v[0], raw[1] = v[1];
+    } else if constexpr (BYTES == 12) {
+      const u3 v = __builtin_amdgcn_raw_buffer_load_b96(rsrc, (int)at, 0, 0);
+      raw[0] = v[0], raw[1] = v[1], raw[2] = v[2];
+    } else {
+      const u4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)at, 0, 0);
+      raw[0] = v[0], raw[1] = v[1], raw[2] = v[2], raw[3] = v[3];
+    }
+    __builtin_memcpy(out, raw, BYTES);
   }
   template <bool VEC>
   __device__ __forceinline__ void store(const T (&in)[Real<T>::VW], unsigned at, unsigned uniform, long col,

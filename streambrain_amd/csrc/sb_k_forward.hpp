@@ -124,48 +124,51 @@ void k_forward(ForwardArgs<T> a) {
   const long nfull = a.N / KC;  // chunks with all KC reduction indices inside the matrix
   SB_PHASE_MARK(0);
   if (VEC) {
-    // per-lane pointers of chunk `w`; every later chunk of this wavefront is NWAVES chunks further on
-    const long rowc = row_ok ? b0 + p : a.B - 1;
-    const T *xp = a.x + rowc * a.N + (long)w * KC + VW * q;
-    const T *wp[VW][NG];
+    // Chunk `w` first; every later chunk of this wavefront is NWAVES chunks further on.  x and W are
+    // reached through bounds-checked buffer windows that start at the chunk (a scalar base address,
+    // advanced with scalar instructions), so the per-lane offsets never change and the loop body is
+    // loads and MFMAs only.  Batch rows past the end and columns past the tile read zero.
+    constexpr unsigned ES = sizeof(T);
+    const T *xbase = a.x + b0 * a.N + (long)w * KC;             // uniform
+    const T *wbase = a.W + (long)w * KC * a.M + j0;             // uniform
+    long xleft = (a.B - b0) * a.N - (long)w * KC;               // elements from xbase to the end of x
+    long wleft = (a.N - (long)w * KC) * a.M - j0;               // ... of W
+    const unsigned xat = (unsigned)(((long)p * a.N + VW * q) * ES);
+    unsigned wat[VW][NG];
 #pragma unroll
     for (int s = 0; s < VW; s++)
 #pragma unroll
-      for (int g = 0; g < NG; g++) {
-        long col = j0 + gcol(g, p);
-        if (col >= jend) col = j0;  // redirected: feeds unused columns only
-        wp[s][g] = a.W + ((long)w * KC + VW * q + s) * a.M + col;
-      }
+      for (int g = 0; g < NG; g++)
+        wat[s][g] = j0 + gcol(g, p) < jend ? (unsigned)(((long)(VW * q + s) * a.M + gcol(g, p)) * ES)
+                                           : BufferWindow<T>::kOutside;
     const long xstep = (long)NWAVES * KC;
     const long wstep = (long)NWAVES * KC * a.M;
     // Chunks w, w + NWAVES, ... < nfull: n of them for this wavefront.  The loop is branch-free: a load
-    // past the last chunk re-reads the last chunk (its pointers stop advancing) and is never used, so
+    // past the last chunk reads whatever lies there (or zeros past the arrays) and is never used, so
     // the compiler can keep exact wait counts and D-1 chunks really are in flight.
     const long n = w < nfull ? (nfull - 1 - w) / NWAVES + 1 : 0;
-    auto load_next = [&](T(&xo)[VW], T(&wo)[VW][NG][VW], bool advance) {
-      const vec_t xv = *reinterpret_cast<const vec_t *>(xp);
-#pragma unroll
-      for (int e = 0; e < VW; e++) xo[e] = xv[e];
-      xp += advance ? xstep : 0;
+    auto load_next = [&](T(&xo)[VW], T(&wo)[VW][NG][VW]) {
+      const BufferWindow<T> xwin(xbase, xleft), wwin(wbase, wleft);
+      xwin.template load_n<VW>(xo, xat);
 #pragma unroll
       for (int s = 0; s < VW; s++)
 #pragma unroll
         for (int g = 0; g < NG; g++) {
           if (gwidth(g) == VW) {
-            const vec_t wv = *reinterpret_cast<const vec_t *>(wp[s][g]);
-#pragma unroll
-            for (int e = 0; e < VW; e++) wo[s][g][e] = wv[e];
+            wwin.template load_n<VW>(wo[s][g], wat[s][g]);
           } else {
-            const PackedCols<T, LW> wv = *reinterpret_cast<const PackedCols<T, LW> *>(wp[s][g]);
+            T t[LW];
+            wwin.template load_n<LW>(t, wat[s][g]);
 #pragma unroll
-            for (int e = 0; e < LW; e++) wo[s][g][e] = wv.v[e];
+            for (int e = 0; e < LW; e++) wo[s][g][e] = t[e];
           }
-          wp[s][g] += advance ? wstep : 0;
         }
+      xbase += xstep, xleft -= xstep;
+      wbase += wstep, wleft -= wstep;
     };
     if (n > 0) {
 #pragma unroll
-      for (int u = 0; u < D - 1; u++) load_next(xr[u], wr[u], u + 1 < n);  // chunks 0 .. D-2
+      for (int u = 0; u < D - 1; u++) load_next(xr[u], wr[u]);  // chunks 0 .. D-2
       __builtin_amdgcn_sched_barrier(0);
       long i = 0;
       for (; i + D <= n; i += D) {
@@ -173,7 +176,7 @@ void k_forward(ForwardArgs<T> a) {
         for (int u = 0; u < D; u++) {
           // the scheduling fences keep the loads where they are written: the compiler's latency model
           // would otherwise sink them to just ahead of their use, far too late for HBM or L2
-          load_next(xr[(u + D - 1) % D], wr[(u + D - 1) % D], i + u + D < n);  // chunk i + u + D - 1
+          load_next(xr[(u + D - 1) % D], wr[(u + D - 1) % D]);  // chunk i + u + D - 1
           __builtin_amdgcn_sched_barrier(0);
           compute(xr[u], wr[u]);                                              // chunk i + u
           __builtin_amdgcn_sched_barrier(0);

@@ -54,6 +54,8 @@ int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias
   SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");
   const long M = H * Mc;
   SB_REQUIRE(M < (1L << 31) && N < (1L << 31), "dimension too large");
+  // per-lane byte offsets inside one chunk of 16 rows of x or W are 32-bit
+  SB_REQUIRE(16 * (N > M ? N : M) * (long)sizeof(T) < (1L << 31), "layer too wide for the forward kernel");
   ForwardArgs<T> a{act, x, W, bias, B, N, M, Mc, 0, cdiv(B, 16)};
   const bool base_vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(W);
   const long need = cdiv(Mc, GW);
