@@ -198,22 +198,22 @@ struct BufferWindow {
     }
   }
   // NE consecutive elements (4, 8, 12 or 16 bytes) as one access; element-aligned
-  template <int NE>
+  template <int NE, int AUX = 0>
   __device__ __forceinline__ void load_n(T (&out)[NE], unsigned at) const {
     constexpr int BYTES = NE * (int)sizeof(T);
     static_assert(BYTES == 4 || BYTES == 8 || BYTES == 12 || BYTES == 16, "one buffer access");
     using u3 = unsigned __attribute__((ext_vector_type(3)));
     unsigned raw[BYTES / 4];
     if constexpr (BYTES == 4) {
-      raw[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)at, 0, 0);
+      raw[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)at, 0, AUX);
     } else if constexpr (BYTES == 8) {
-      const u2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)at, 0, 0);
+      const u2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)at, 0, AUX);
       raw[0] = v[0], raw[1] = v[1];
     } else if constexpr (BYTES == 12) {
-      const u3 v = __builtin_amdgcn_raw_buffer_load_b96(rsrc, (int)at, 0, 0);
+      const u3 v = __builtin_amdgcn_raw_buffer_load_b96(rsrc, (int)at, 0, AUX);
       raw[0] = v[0], raw[1] = v[1], raw[2] = v[2];
     } else {
-      const u4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)at, 0, 0);
+      const u4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)at, 0, AUX);
       raw[0] = v[0], raw[1] = v[1], raw[2] = v[2], raw[3] = v[3];
     }
     __builtin_memcpy(out, raw, BYTES);

@@ -86,7 +86,7 @@ void k_forward(ForwardArgs<T> a) {
     for (int c = 0; c < VW; c++) acc[g][c] = acc_t{0, 0, 0, 0};
 
   // ring of D chunk buffers: D-1 chunks of loads are in flight while one is being multiplied
-  constexpr int D = NG <= 2 ? 3 : 2;
+  constexpr int D = 2;  // measured: deeper rings are slower, the CU cannot keep more loads in flight anyway
   T xr[D][VW];
   T wr[D][VW][NG][VW];
 
@@ -121,6 +121,16 @@ void k_forward(ForwardArgs<T> a) {
     }
   };
 
+  // the epilogue's bias values (thread tid < 256: batch row tid / 16, columns tid % 16 + 16 t) are
+  // requested before the K loop, so their latency is not added to the epilogue
+  constexpr int PER = NG * VW;
+  const long ncol = jend - j0;
+  T bv[PER];
+#pragma unroll
+  for (int t = 0; t < PER; t++) {
+    const long col = (tid & 15) + 16 * t;
+    bv[t] = a.bias[j0 + (col < ncol ? col : 0)];
+  }
   const long nfull = a.N / KC;  // chunks with all KC reduction indices inside the matrix
   SB_PHASE_MARK(0);
   if (VEC) {
@@ -247,16 +257,8 @@ void k_forward(ForwardArgs<T> a) {
   // ---- bias (+ softmax): 16 threads per batch row (256 threads), thread handles columns l16 + 16 t
   if (tid >= 256) return;
   const int row = tid >> 4, l16 = tid & 15;
-  const long ncol = jend - j0;
-  constexpr int PER = NG * VW;
   T vals[PER];
   T mx = -INFINITY;
-  T bv[PER];
-#pragma unroll
-  for (int t = 0; t < PER; t++) {  // branch-free, so the loads are in flight together
-    const long col = l16 + 16 * t;
-    bv[t] = a.bias[j0 + (col < ncol ? col : 0)];
-  }
 #pragma unroll
   for (int t = 0; t < PER; t++) {
     const long col = l16 + 16 * t;
