@@ -15,8 +15,8 @@
 //      "k-major" in memory, which is the 16x16x4 MFMA operand layout, so staging is a plain copy and
 //      each wavefront feeds its 32 x 32 sub-tile (2 x 2 MFMA blocks) with two 8-byte LDS reads per K
 //      step of 4.  The global loads of chunk c+1 are issued before chunk c is consumed.
-//   2. From the same LDS slabs, 32 lanes of each wavefront add up one column each of x (resp. y) in
-//      batch order b = 0..B-1 without FMA contraction: the reference's summation order, so Ci, Cj and
+//   2. From the same LDS slabs, the lanes of one wavefront add up one column each of x, those of
+//      another one column each of y, in batch order b = 0..B-1 without FMA contraction: the reference's summation order, so Ci, Cj and
 //      kbi stay bit-exact against a strict-IEEE build of it.  Every tile needs Ci for its rows and Cj
 //      for its columns, so every workgroup recomputes them from the OLD traces (a tile row shares x,
 //      a tile column shares y: same inputs, same order, same bits).  The old traces are read from
@@ -128,10 +128,13 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   };
   request_chunk(0);
 
-  // column sums: lanes 0..31 of wavefronts 0,1 take the 64 x columns, of wavefronts 2,3 the y columns
-  const bool summer = lane < 32;
-  const bool sum_i = w < 2;
-  const int scol = (w & 1) * 32 + (lane & 31);
+  // column sums: one wavefront takes the 64 x columns of the tile (a lane each), one the 64 y columns,
+  // the other two take none; which wavefronts do rotates with the tile, so that over the tiles of a
+  // CU the work is spread over its four SIMDs
+  const int role = __builtin_amdgcn_readfirstlane((w + (int)tile) & 3);
+  const bool summer = role < 2;  // uniform per wavefront
+  const bool sum_i = role == 0;
+  const int scol = lane;
   const T *sbase = (sum_i ? xs : ys) + scol;
   const long sidx = (sum_i ? i0 : j0) + scol;
   const bool sum_ok = summer && sidx < (sum_i ? a.N : a.M);
