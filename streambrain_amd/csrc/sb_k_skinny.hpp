@@ -1,0 +1,125 @@
+// Layers with very few output units (the 10-unit classification layer): forward and training passes on
+// plain vector arithmetic.  With M <= 32 output columns an MFMA tile would be mostly padding, and the
+// whole problem is a few million multiply-adds whose cost is latency, not arithmetic; what matters is
+// that every load is coalesced and that no thread does more than a few hundred instructions.
+//
+// Thread layout shared by both kernels: R = 256 / M rows of W (or Cij) per pass, thread t < R*M owns
+// column j = t % M of row r = t / M, so the R*M threads of a pass read R*M consecutive elements.
+#pragma once
+#include "sb_kernels.hpp"
+
+namespace sb {
+
+// act[b, :] = softmax_per_hypercolumn(x[b, :] . W + bias)      omp.cc:70-87 + kernels_numpy.py:13-25
+// One workgroup per batch row.  Partial sums over the rows r, r + R, ... are added up in the order of r
+// (fixed, so the result is deterministic).
+template <typename T>
+__global__ __launch_bounds__(256) void k_forward_skinny(T *act, const T *x, const T *W, const T *bias,
+                                                        long N, long M, long Mc, int softmax) {
+  __shared__ T part[256];
+  __shared__ T logit[32];
+  const int tid = threadIdx.x;
+  const int R = 256 / (int)M;
+  const int j = tid % (int)M, r = tid / (int)M;
+  const T *xrow = x + (long)blockIdx.x * N;
+  T acc = T(0);
+  if (r < R) {
+    // pointers advance by R rows per step, so a load costs one address addition and no multiplication
+    const T *xq = xrow + r, *wq = W + (long)r * M + j;
+    const long wstep = (long)R * M;
+    long i = r;
+    for (; i + 7 * R < N; i += 8 * R) {  // 8 rows of loads in flight
+      T xv[8], wv[8];
+#pragma unroll
+      for (int k = 0; k < 8; k++) {
+        xv[k] = *xq, wv[k] = *wq;
+        xq += R, wq += wstep;
+      }
+#pragma unroll
+      for (int k = 0; k < 8; k++) acc += xv[k] * wv[k];
+    }
+    for (; i < N; i += R, xq += R, wq += wstep) acc += *xq * *wq;
+  }
+  part[tid] = acc;
+  __syncthreads();
+  if (tid < M) {
+    T s = T(0);
+    for (int k = 0; k < R; k++) s += part[k * (int)M + tid];
+    logit[tid] = s + bias[tid];
+  }
+  __syncthreads();
+  if (tid < M) {
+    T v = logit[tid];
+    if (softmax) {
+      const int h0 = (tid / (int)Mc) * (int)Mc;  // first unit of this thread's hypercolumn
+      T mx = -INFINITY;
+      for (int c = 0; c < Mc; c++) mx = logit[h0 + c] > mx ? logit[h0 + c] : mx;
+      T sum = T(0);
+      for (int c = 0; c < Mc; c++) sum += Real<T>::exp_(logit[h0 + c] - mx);
+      v = Real<T>::exp_(v - mx) / sum;
+    }
+    act[(long)blockIdx.x * M + tid] = v;
+  }
+}
+
+// The fused training pass of k_train_fused (same arguments, same results within rounding) for M <= 32:
+// one workgroup per R rows of Cij; thread (r, j) walks the batch once, accumulating its x^T y element
+// and, in batch order and without FMA contraction, the column sums its row's Ci and its column's Cj
+// are made of -- the reference's order, so the traces are bit-exact as in the tiled kernel.
+template <typename T>
+__global__ __launch_bounds__(256) void k_train_skinny(TrainArgs<T> a) {
+  using Rl = Real<T>;
+  const int tid = threadIdx.x;
+  const int M = (int)a.M;
+  const int R = 256 / M;
+  const int j = tid % M, r = tid / M;
+  const long i = (long)blockIdx.x * R + r;
+  if (r >= R || i >= a.N) return;  // no barriers below
+  T dot = T(0), sx = T(0), sy = T(0);
+  const T *xp = a.x + i, *yp = a.y + j;
+  // 16 batch rows of loads in flight (branch-free: past the batch the last row is re-read and counts
+  // as 0), then the ordered arithmetic; the pointers advance by one row per load
+  for (long b0 = 0; b0 < a.B; b0 += 16) {
+    T xv[16], yv[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+      const bool live = b0 + k < a.B;  // uniform; the pointers stop at the last row of the batch
+      xv[k] = *xp, yv[k] = *yp;
+      xp += live && b0 + k + 1 < a.B ? a.N : 0;
+      yp += live && b0 + k + 1 < a.B ? a.M : 0;
+    }
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+      const bool live = b0 + k < a.B;
+      const T xk = live ? xv[k] : T(0), yk = live ? yv[k] : T(0);
+      dot += xk * yk;
+      sx = Rl::add(sx, xk);
+      sy = Rl::add(sy, yk);
+    }
+  }
+  auto trace = [&](T cold, T sum) {
+    T s = Rl::div(sum, a.fB);
+    s = Rl::mul(s, a.tau);
+    const T c = Rl::add(Rl::mul(cold, a.omt), s);
+    return c > T(0) ? c : T(0);
+  };
+  const T ci = trace(a.Ci[i], sx), cj = trace(a.Cj[j], sy);
+  if (j == 0) a.Ci_next[i] = ci;
+  if (i == 0) {
+    a.Cj_next[j] = cj;
+    if (a.bias_mode == 1) {
+      T kb = a.kbi[j];
+      a.bias[j] = bias_regularized<T>(cj, kb, a.cthr, a.khalf, a.pmin, a.taubdt);
+      a.kbi[j] = kb;
+    }
+  }
+  T cn = a.Cij[i * a.M + j] * a.omt + dot * (a.invB * a.tau);
+  cn = fmax(cn, T(0));
+  a.Cij[i * a.M + j] = cn;
+  const T wgt = weight_from_traces<T>(cn, trace_reciprocal<T>(ci, a.cthr), trace_reciprocal<T>(cj, a.cthr),
+                                      a.cthr4);
+  const bool on = a.wmask == nullptr || a.wmask[i * a.H + j / (int)a.Mc] != 0;
+  a.W[i * a.M + j] = on ? wgt : T(0);
+}
+
+}  // namespace sb

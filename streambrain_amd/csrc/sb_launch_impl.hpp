@@ -3,6 +3,7 @@
 #pragma once
 #include "sb_kernels.hpp"
 #include "sb_k_train.hpp"
+#include "sb_k_skinny.hpp"
 #include "sb_launch.hpp"
 
 #include <cstdlib>
@@ -54,6 +55,14 @@ int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias
   SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");
   const long M = H * Mc;
   SB_REQUIRE(M < (1L << 31) && N < (1L << 31), "dimension too large");
+  if (M <= 32) {  // a handful of output units: plain vector arithmetic, one workgroup per batch row
+    SB_REQUIRE(B < (1L << 31), "batch too large for one launch");
+    ProfScope prof_(st, K_FORWARD);
+    hipLaunchKernelGGL((k_forward_skinny<T>), dim3((unsigned)B), dim3(256), 0, st, act, x, W, bias, N, M, Mc,
+                       softmax ? 1 : 0);
+    SB_LAUNCH_CHECK();
+    return 0;
+  }
   // per-lane byte offsets inside one chunk of 16 rows of x or W are 32-bit
   SB_REQUIRE(16 * (N > M ? N : M) * (long)sizeof(T) < (1L << 31), "layer too wide for the forward kernel");
   ForwardArgs<T> a{act, x, W, bias, B, N, M, Mc, 0, cdiv(B, 16)};
@@ -123,6 +132,14 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   a.tau = s.tau; a.omt = s.omt; a.fB = (T)B; a.invB = (T)1 / (T)B; a.cthr = s.cthr; a.cthr4 = s.cthr4;
   a.khalf = khalf; a.pmin = pmin; a.taubdt = taubdt;
   a.tiles_i = cdiv(N, 64); a.tiles_j = cdiv(M, 64);
+  if (M <= 32) {  // a handful of output units: plain vector arithmetic
+    const long rows = 256 / M;
+    SB_REQUIRE(cdiv(N, rows) < (1L << 31), "too many rows for one launch");
+    ProfScope prof_(st, K_TRAIN_FUSED);
+    hipLaunchKernelGGL((k_train_skinny<T>), dim3((unsigned)cdiv(N, rows)), dim3(256), 0, st, a);
+    SB_LAUNCH_CHECK();
+    return 0;
+  }
   SB_REQUIRE(a.tiles_i * a.tiles_j < (1L << 31) - 8, "too many tiles for one launch");
   // the kernel addresses x, y and one 64-row band of Cij / W through 32-bit buffer windows of 2 GiB
   SB_REQUIRE((B + 64) * (N > M ? N : M) * (long)sizeof(T) <= (1L << 31),
