@@ -107,11 +107,10 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   // return in issue order, hence the order below: first what the first MFMA needs (chunk 0 of x and
   // y, mostly L2 hits), and the Cij tile (HBM) only while the second-to-last chunk is being computed.
   constexpr unsigned ES = sizeof(T);
-  const BufferWindow<T> xwin(a.x, a.B * a.N), ywin(a.y, a.B * a.M);
   const long tile_rows = a.N - i0 < TS ? a.N - i0 : TS;
   const BufferWindow<T> cwin(a.Cij + i0 * a.M, tile_rows * a.M), wwin(a.W + i0 * a.M, tile_rows * a.M);
   T sx[SP][VW], sy[SP][VW];
-  // byte offsets of this thread's vectors in chunk 0; chunk c is c * KCH rows further on
+  // byte offsets of this thread's vectors relative to the first row of a chunk
   unsigned xat[SP], yat[SP];
 #pragma unroll
   for (int m = 0; m < SP; m++) {
@@ -119,11 +118,13 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
     yat[m] = (unsigned)(((long)(er + RPP * m) * a.M + ecol) * ES);
   }
   auto request_chunk = [&](long b0) {
-    const unsigned xrow = (unsigned)(b0 * a.N * ES), yrow = (unsigned)(b0 * a.M * ES);
+    // windows from the chunk's first batch row to the end of x / y (scalar arithmetic): rows past the
+    // batch fall outside, and the per-lane offsets stay those of chunk 0 whatever the batch size
+    const BufferWindow<T> xwin(a.x + b0 * a.N, (a.B - b0) * a.N), ywin(a.y + b0 * a.M, (a.B - b0) * a.M);
 #pragma unroll
     for (int m = 0; m < SP; m++) {
-      xwin.template load<VEC>(sx[m], xat[m], xrow, i0 + VW * eg, a.N);
-      ywin.template load<VEC>(sy[m], yat[m], yrow, ecol, a.M);
+      xwin.template load<VEC>(sx[m], xat[m], 0, i0 + VW * eg, a.N);
+      ywin.template load<VEC>(sy[m], yat[m], 0, ecol, a.M);
     }
   };
   request_chunk(0);

@@ -141,10 +141,10 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
     return 0;
   }
   SB_REQUIRE(a.tiles_i * a.tiles_j < (1L << 31) - 8, "too many tiles for one launch");
-  // the kernel addresses x, y and one 64-row band of Cij / W through 32-bit buffer windows of 2 GiB
-  SB_REQUIRE((B + 64) * (N > M ? N : M) * (long)sizeof(T) <= (1L << 31),
-             "batch too large: batch rows x layer width must stay below 2 GiB");
-  SB_REQUIRE(64 * M * (long)sizeof(T) <= (1L << 31), "layer too wide: 64 rows of Cij must stay below 2 GiB");
+  // the kernel addresses a chunk of x and y rows and one 64-row band of Cij / W through buffer windows
+  // with 32-bit offsets
+  SB_REQUIRE(64 * (N > M ? N : M) * (long)sizeof(T) <= (1L << 31),
+             "layer too wide: 64 rows of it must stay below 2 GiB");
   const bool vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(y) && aligned16(Cij) &&
                    aligned16(W);
   // 8 workgroup ids per round of XCDs; ids beyond the last tile exit at once
