@@ -79,6 +79,21 @@ int sb_compute_activation_f32(float *d_act, const float *d_x, const float *d_W,
 int sb_compute_activation_f64(double *d_act, const double *d_x, const double *d_W,
                               const double *d_bias, long B, long N, long H, long Mc);
 
+/* compute_activation for a masked layer: W must be zero wherever wmask is 0 (the state apply_mask,
+ * kernels_openmp_internal.cc:322-335, leaves behind), and the reduction then runs over the connected
+ * rows only.  sb_mask_rows builds what it needs from wmask[N,H]: d_rows[H,cap] = ascending indices
+ * of the set bytes of each column, then -1 up to cap (cap: a multiple of 16, at least
+ * the largest column count rounded up), d_row_cnt[H] = the column counts.  Same result as
+ * sb_compute_activation on such a W, up to the order of the sum.  Needs Mc and H*Mc divisible by 4
+ * (f32) or 2 (f64), Mc <= 256 (f32) or 224 (f64), 16-byte aligned W. */
+int sb_mask_rows(int *d_rows, int *d_row_cnt, const unsigned char *d_wmask, long N, long H, long cap);
+int sb_compute_activation_rows_f32(float *d_act, const float *d_x, const float *d_W,
+                                   const float *d_bias, const int *d_rows, const int *d_row_cnt,
+                                   long cap, long B, long N, long H, long Mc);
+int sb_compute_activation_rows_f64(double *d_act, const double *d_x, const double *d_W,
+                                   const double *d_bias, const int *d_rows, const int *d_row_cnt,
+                                   long cap, long B, long N, long H, long Mc);
+
 /* Ci, Cj, Cij moving averages (clamped at 0) and W = log(max(Cij,cthr^4)/(Ci*Cj)) with rows
  * Ci<cthr and columns Cj<cthr zeroed; all in place; W is the unmasked weight.
  * replaces update_weights_float32/64 -> vectorized_updateWeights,

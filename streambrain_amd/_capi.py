@@ -22,6 +22,7 @@ _KERNEL_SIGS = {
     "sb_update_state": lambda R: [_P, _P, _P, _P, _L, _L, _L],
     "sb_softmax_minicolumns": lambda R: [_P, _L, _L, _L],
     "sb_compute_activation": lambda R: [_P, _P, _P, _P, _L, _L, _L, _L],
+    "sb_compute_activation_rows": lambda R: [_P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _L],
     "sb_update_weights": lambda R: [_P, _P, _P, _P, _P, R, _P, R, _L, _L, _L],
     "sb_update_bias": lambda R: [_P, _P, R, _L],
     "sb_update_bias_regularized": lambda R: [_P, _P, _P, R, R, R, R, _L],
@@ -42,6 +43,7 @@ _PLAIN_SIGS = {
     "sb_memcpy_d2h": [_P, _P, _Z],
     "sb_memcpy_d2d": [_P, _P, _Z],
     "sb_fill_bytes": [_P, _I, _Z],
+    "sb_mask_rows": [_P, _P, _P, _L, _L, _L],
     "sb_net_create": [ctypes.POINTER(_P), _I],
     "sb_net_destroy": [_P],
     "sb_net_add_dense_layer": [_P, _L, _L, _L, _D, _D, _D, _D],

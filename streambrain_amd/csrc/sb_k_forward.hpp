@@ -35,6 +35,127 @@ struct ForwardArgs {
   long col_tiles, batch_tiles;
 };
 
+// Column layout of a tile, shared by the kernels below: NG groups of 16 lanes-columns, group g holding
+// VW column blocks (the last group LW <= VW), lane p of a group owning gwidth(g) consecutive columns.
+template <typename T, int NG, int LW>
+struct TileCols {
+  static constexpr int VW = Real<T>::VW;
+  static constexpr int GW = 16 * VW;
+  static constexpr int CP = NG * GW + VW;  // padded row length of a tile in LDS
+  __device__ static constexpr int gwidth(int g) { return g == NG - 1 ? LW : VW; }
+  __device__ static constexpr int gcol(int g, int p) { return g * GW + gwidth(g) * p; }
+};
+
+template <typename T, int LW>
+struct PackedCols {  // LW consecutive elements, element-aligned
+  T v[LW];
+} __attribute__((packed, aligned(sizeof(T))));
+
+// Tail of the forward kernels: the NWAVES partial tiles (one per wavefront, in MFMA accumulator layout)
+// are summed through LDS in a fixed order (deterministic), then 16 threads per batch row add the bias
+// and, when FUSE, do the softmax over the tile's ncol columns.  bv: the bias values of thread tid < 256
+// (columns tid % 16 + 16 t), loaded by the caller ahead of its main loop.
+template <typename T, int NG, bool FUSE, int NWAVES, int LW>
+__device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&acc)[NG][Real<T>::VW],
+                                               const T (&bv)[NG * Real<T>::VW],
+                                               T (&red)[NWAVES / 2][16][TileCols<T, NG, LW>::CP], T *act,
+                                               long B, long M, long b0, long j0, long ncol) {
+  using TC = TileCols<T, NG, LW>;
+  constexpr int VW = Real<T>::VW;
+  constexpr int PER = NG * VW;
+  using vec_t = typename Real<T>::vec_t;
+  auto gwidth = [](int g) { return TC::gwidth(g); };
+  auto gcol = [](int g, int p_) { return TC::gcol(g, p_); };
+  const int tid = threadIdx.x, lane = tid & 63, p = lane & 15, q = lane >> 4;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // ---- cross-wavefront sum through LDS in a fixed order (deterministic): the upper half of the
+  // wavefronts hands its partial tiles over, the lower half adds them to its own and publishes the
+  // sums (each lane rewrites exactly the elements it has just read, so no barrier is needed between
+  // the two); the row-wise epilogue then adds up the HALF published tiles.
+  constexpr int HALF = NWAVES / 2;
+  static_assert(NWAVES >= 2 && (NWAVES & (NWAVES - 1)) == 0, "a power of two, at least 2 wavefronts");
+  if (w >= HALF) {
+#pragma unroll
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        T *slot = &red[w - HALF][Real<T>::acc_row(q, v)][gcol(g, p)];
+        if (gwidth(g) == VW) {
+          vec_t t;
+#pragma unroll
+          for (int c = 0; c < VW; c++) t[c] = acc[g][c][v];
+          *reinterpret_cast<vec_t *>(slot) = t;
+        } else {
+#pragma unroll
+          for (int c = 0; c < LW; c++) slot[c] = acc[g][c][v];
+        }
+      }
+  }
+  __syncthreads();
+  if (w < HALF) {
+#pragma unroll
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        T *slot = &red[w][Real<T>::acc_row(q, v)][gcol(g, p)];
+        if (gwidth(g) == VW) {
+          vec_t t = *reinterpret_cast<vec_t *>(slot);
+#pragma unroll
+          for (int c = 0; c < VW; c++) t[c] += acc[g][c][v];
+          *reinterpret_cast<vec_t *>(slot) = t;
+        } else {
+#pragma unroll
+          for (int c = 0; c < LW; c++) slot[c] += acc[g][c][v];
+        }
+      }
+  }
+  __syncthreads();
+
+  SB_PHASE_MARK(2);
+  // ---- bias (+ softmax): 16 threads per batch row (256 threads), thread handles columns l16 + 16 t
+  if (tid >= 256) return;
+  const int row = tid >> 4, l16 = tid & 15;
+  T vals[PER];
+  T mx = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < PER; t++) {
+    const long col = l16 + 16 * t;
+    T sum = red[0][row][col < ncol ? col : 0];
+#pragma unroll
+    for (int h = 1; h < HALF; h++) sum += red[h][row][col < ncol ? col : 0];
+    vals[t] = col < ncol ? sum + bv[t] : T(0);
+    mx = (col < ncol && vals[t] > mx) ? vals[t] : mx;
+  }
+  if (FUSE) {
+#pragma unroll
+    for (int o = 8; o >= 1; o >>= 1) {
+      const T other = __shfl_xor(mx, o);
+      mx = other > mx ? other : mx;
+    }
+    T sum = T(0);
+#pragma unroll
+    for (int t = 0; t < PER; t++) {
+      const long col = l16 + 16 * t;
+      if (col < ncol) {
+        vals[t] = Real<T>::exp_(vals[t] - mx);
+        sum += vals[t];
+      }
+    }
+#pragma unroll
+    for (int o = 8; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+#pragma unroll
+    for (int t = 0; t < PER; t++) vals[t] = vals[t] / sum;
+  }
+  if (b0 + row < B) {
+    T *out = act + (b0 + row) * M + j0;
+#pragma unroll
+    for (int t = 0; t < PER; t++) {
+      const long col = l16 + 16 * t;
+      if (col < ncol) out[col] = vals[t];
+    }
+  }
+}
+
 // Unguarded 16-byte loads of the main loop: rows / columns outside the matrix are redirected to a valid
 // address (their products land in accumulator rows / columns that are never stored), so the loop body
 // is loads + MFMAs + pointer bumps only.  The last, partial K chunk takes the guarded path.
@@ -45,11 +166,6 @@ struct ForwardArgs {
 // 8: with LW = 3 the last group's lanes load LW consecutive columns (12 bytes) instead of VW, and a
 // quarter of that group's MFMAs disappears.  The launcher picks LW < VW only when no vector of the last
 // group straddles the end of the tile.
-template <typename T, int LW>
-struct PackedCols {  // LW consecutive elements, element-aligned
-  T v[LW];
-} __attribute__((packed, aligned(sizeof(T))));
-
 template <typename T, int NG, bool FUSE, bool VEC, int NWAVES, int LW = Real<T>::VW>
 __global__ __launch_bounds__(64 * NWAVES) __attribute__((amdgpu_waves_per_eu(NWAVES / 4, NWAVES / 4)))
 void k_forward(ForwardArgs<T> a) {
@@ -210,92 +326,7 @@ void k_forward(ForwardArgs<T> a) {
   }
 
   SB_PHASE_MARK(1);
-  // ---- cross-wavefront sum through LDS in a fixed order (deterministic): the upper half of the
-  // wavefronts hands its partial tiles over, the lower half adds them to its own and publishes the
-  // sums (each lane rewrites exactly the elements it has just read, so no barrier is needed between
-  // the two); the row-wise epilogue then adds up the HALF published tiles.
-  constexpr int HALF = NWAVES / 2;
-  static_assert(NWAVES >= 2 && (NWAVES & (NWAVES - 1)) == 0, "a power of two, at least 2 wavefronts");
-  if (w >= HALF) {
-#pragma unroll
-    for (int g = 0; g < NG; g++)
-#pragma unroll
-      for (int v = 0; v < 4; v++) {
-        T *slot = &red[w - HALF][Real<T>::acc_row(q, v)][gcol(g, p)];
-        if (gwidth(g) == VW) {
-          vec_t t;
-#pragma unroll
-          for (int c = 0; c < VW; c++) t[c] = acc[g][c][v];
-          *reinterpret_cast<vec_t *>(slot) = t;
-        } else {
-#pragma unroll
-          for (int c = 0; c < LW; c++) slot[c] = acc[g][c][v];
-        }
-      }
-  }
-  __syncthreads();
-  if (w < HALF) {
-#pragma unroll
-    for (int g = 0; g < NG; g++)
-#pragma unroll
-      for (int v = 0; v < 4; v++) {
-        T *slot = &red[w][Real<T>::acc_row(q, v)][gcol(g, p)];
-        if (gwidth(g) == VW) {
-          vec_t t = *reinterpret_cast<vec_t *>(slot);
-#pragma unroll
-          for (int c = 0; c < VW; c++) t[c] += acc[g][c][v];
-          *reinterpret_cast<vec_t *>(slot) = t;
-        } else {
-#pragma unroll
-          for (int c = 0; c < LW; c++) slot[c] += acc[g][c][v];
-        }
-      }
-  }
-  __syncthreads();
-
-  SB_PHASE_MARK(2);
-  // ---- bias (+ softmax): 16 threads per batch row (256 threads), thread handles columns l16 + 16 t
-  if (tid >= 256) return;
-  const int row = tid >> 4, l16 = tid & 15;
-  T vals[PER];
-  T mx = -INFINITY;
-#pragma unroll
-  for (int t = 0; t < PER; t++) {
-    const long col = l16 + 16 * t;
-    T sum = red[0][row][col < ncol ? col : 0];
-#pragma unroll
-    for (int h = 1; h < HALF; h++) sum += red[h][row][col < ncol ? col : 0];
-    vals[t] = col < ncol ? sum + bv[t] : T(0);
-    mx = (col < ncol && vals[t] > mx) ? vals[t] : mx;
-  }
-  if (FUSE) {
-#pragma unroll
-    for (int o = 8; o >= 1; o >>= 1) {
-      const T other = __shfl_xor(mx, o);
-      mx = other > mx ? other : mx;
-    }
-    T sum = T(0);
-#pragma unroll
-    for (int t = 0; t < PER; t++) {
-      const long col = l16 + 16 * t;
-      if (col < ncol) {
-        vals[t] = Real<T>::exp_(vals[t] - mx);
-        sum += vals[t];
-      }
-    }
-#pragma unroll
-    for (int o = 8; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
-#pragma unroll
-    for (int t = 0; t < PER; t++) vals[t] = vals[t] / sum;
-  }
-  if (b0 + row < a.B) {
-    T *out = a.act + (b0 + row) * a.M + j0;
-#pragma unroll
-    for (int t = 0; t < PER; t++) {
-      const long col = l16 + 16 * t;
-      if (col < ncol) out[col] = vals[t];
-    }
-  }
+  forward_finish<T, NG, FUSE, NWAVES, LW>(acc, bv, red, a.act, a.B, a.M, b0, j0, ncol);
   SB_PHASE_MARK(3);
 }
 

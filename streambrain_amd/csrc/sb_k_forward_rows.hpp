@@ -1,0 +1,205 @@
+// Forward pass of a structural-plasticity layer over the connected inputs only.
+//
+// The layer keeps W masked (apply_mask, omp.cc:322-335): W[i, columns of hypercolumn h] is zero
+// wherever wmask[i, h] is 0, so in  act = softmax_per_hypercolumn(x . W + bias)  (omp.cc:70-87 +
+// kernels_numpy.py:13-25) those rows add exact zeros to hypercolumn h.  With a connection density of
+// 0.1 nine tenths of the reduction are such zeros.  k_forward_rows skips them: per hypercolumn it walks
+// the ascending list of connected rows (k_mask_rows keeps the lists in step with wmask) and gathers
+// those rows of W and those columns of x.  Same tiling, accumulator layout and epilogue as k_forward.
+#pragma once
+#include "sb_k_forward.hpp"
+
+namespace sb {
+
+// rows[h * cap + 0 .. cnt_h) = ascending indices i with wmask[i, h] != 0, the rest of the cap entries
+// -1; row_cnt[h] = cnt_h.  One workgroup per hypercolumn h0 + blockIdx.x; entries beyond
+// `cap` are dropped (the host sizes cap from the column counts, so none are).  (A template only so that
+// the header can be included from several translation units.)
+template <int = 0>
+__global__ __launch_bounds__(256) void k_mask_rows(int *rows, int *row_cnt, const uint8_t *wmask, long N,
+                                                   long H, long cap, long h0) {
+  __shared__ int scan[256];
+  const int tid = threadIdx.x;
+  const long h = h0 + blockIdx.x;
+  const long seg = (N + 255) / 256;
+  const long lo = tid * seg < N ? tid * seg : N, hi = lo + seg < N ? lo + seg : N;
+  int mine = 0;
+  for (long i = lo; i < hi; i++) mine += wmask[i * H + h] != 0;
+  scan[tid] = mine;
+  __syncthreads();
+  for (int o = 1; o < 256; o <<= 1) {  // inclusive scan of the per-thread counts
+    const int other = tid >= o ? scan[tid - o] : 0;
+    __syncthreads();
+    scan[tid] += other;
+    __syncthreads();
+  }
+  int *list = rows + h * cap;
+  long pos = scan[tid] - mine;
+  for (long i = lo; i < hi; i++)
+    if (wmask[i * H + h] != 0) {
+      if (pos < cap) list[pos] = (int)i;
+      pos++;
+    }
+  const long total = scan[255] < cap ? scan[255] : cap;
+  for (long k = total + tid; k < cap; k += 256) list[k] = -1;
+  if (tid == 0) row_cnt[h] = (int)total;
+}
+
+template <typename T>
+struct ForwardRowsArgs {
+  ForwardArgs<T> f;
+  const int *rows;     // [H, cap], see k_mask_rows
+  const int *row_cnt;  // [H]
+  long cap;            // a multiple of 16
+};
+
+// A workgroup owns 16 batch rows x one hypercolumn (as k_forward with FUSE).  The hypercolumn's row list
+// is staged through LDS in segments of SEG entries; the wavefronts split a segment in interleaved chunks
+// of 4*VW entries.  Per chunk, lane (p,q) reads the VW list entries VW*q .. VW*q+VW-1 from LDS, then
+// x[b0+p, row] for each of them (the A operands of VW MFMA steps) and VW*NG vectors of VW columns of
+// W[row, :] (the B operands); the operands of one chunk are in flight while the previous one is
+// multiplied.  A padding entry (-1) contributes x = 0 times row 0 of W.  Nothing up to the first MFMAs
+// depends on the hypercolumn's row count: every wavefront multiplies its first chunk of the first
+// segment, which is padding where the list is shorter.
+// Requires M % VW == 0, Mc % VW == 0 and 16-byte aligned W.
+template <typename T, int NG, int NWAVES>
+__global__ __launch_bounds__(64 * NWAVES) __attribute__((amdgpu_waves_per_eu(NWAVES / 4, NWAVES / 4)))
+void k_forward_rows(ForwardRowsArgs<T> ar) {
+  const ForwardArgs<T> &a = ar.f;
+  constexpr int VW = Real<T>::VW;
+  using TC = TileCols<T, NG, VW>;
+  constexpr int KC = 4 * VW;      // list entries per chunk
+  constexpr int SEG = 2048;       // list entries per segment
+  constexpr int SEGC = SEG / KC;  // chunks per segment
+  static_assert(SEGC >= NWAVES && SEG % (64 * NWAVES) == 0, "segment size");
+  using acc_t = typename Real<T>::acc_t;
+  using vec_t = typename Real<T>::vec_t;
+  typedef int ivec_t __attribute__((ext_vector_type(VW)));
+  __shared__ __attribute__((aligned(16))) T red[NWAVES / 2][16][TC::CP];
+  __shared__ __attribute__((aligned(16))) int sidx[SEG];
+
+  // XCD-aware renumbering, as in k_forward
+  const long ntiles = a.col_tiles * a.batch_tiles;
+  const long per_xcd = (ntiles + 7) / 8;
+  const long tile = (long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (tile >= ntiles) return;  // whole workgroup, before any barrier
+  const long ct = tile / a.batch_tiles, bt = tile % a.batch_tiles;
+
+  const int tid = threadIdx.x, lane = tid & 63, p = lane & 15, q = lane >> 4;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const long b0 = bt * 16;
+  const long j0 = ct * a.Mc;
+  const long ncol = a.Mc;
+  const int *list = ar.rows + ct * ar.cap;
+  SB_PHASE_MARK(0);
+
+  // first segment of the list on its way before anything else
+  constexpr int PT = SEG / (64 * NWAVES);  // entries per thread and segment
+  int mine[PT];
+  auto request_segment = [&](long seg0) {
+#pragma unroll
+    for (int t = 0; t < PT; t++) {
+      const long k = seg0 + tid + t * (64 * NWAVES);
+      mine[t] = list[k < ar.cap ? k : 0];  // entries past the list are replaced by padding below
+    }
+  };
+  auto publish_segment = [&](long seg0) {
+#pragma unroll
+    for (int t = 0; t < PT; t++) {
+      const long k = seg0 + tid + t * (64 * NWAVES);
+      sidx[tid + t * (64 * NWAVES)] = k < ar.cap ? mine[t] : -1;
+    }
+  };
+  request_segment(0);
+  const int cnt = ar.row_cnt[ct];
+
+  acc_t acc[NG][VW];
+#pragma unroll
+  for (int g = 0; g < NG; g++)
+#pragma unroll
+    for (int c = 0; c < VW; c++) acc[g][c] = acc_t{0, 0, 0, 0};
+
+  constexpr int PER = NG * VW;
+  T bv[PER];
+#pragma unroll
+  for (int t = 0; t < PER; t++) {
+    const long col = (tid & 15) + 16 * t;
+    bv[t] = a.bias[j0 + (col < ncol ? col : 0)];
+  }
+
+  // x through a bounds-checked window over this tile's 16 batch rows: rows past the batch and padding
+  // entries (offset kOutside) read zero
+  const BufferWindow<T> xwin(a.x + b0 * a.N, (a.B - b0) * a.N);
+  const unsigned xat = (unsigned)((long)p * a.N * sizeof(T));
+  // W: this lane's columns of group g, or the tile's first columns where the group hangs over the end
+  // of the hypercolumn (those accumulator columns are never stored)
+  const T *wcol[NG];
+#pragma unroll
+  for (int g = 0; g < NG; g++) wcol[g] = a.W + j0 + (TC::gcol(g, p) < ncol ? TC::gcol(g, p) : 0);
+
+  T xr[2][VW];
+  T wr[2][VW][NG][VW];
+  // operands of chunk c of the staged segment (c past the segment: its last chunk again, never used)
+  auto request = [&](int c, T(&xo)[VW], T(&wo)[VW][NG][VW]) {
+    const ivec_t idx = *reinterpret_cast<const ivec_t *>(&sidx[(c < SEGC ? c : SEGC - 1) * KC + VW * q]);
+#pragma unroll
+    for (int s = 0; s < VW; s++) {
+      const int r = idx[s];
+      T one[1];
+      xwin.template load_n<1>(one, r < 0 ? BufferWindow<T>::kOutside : xat + (unsigned)r * (unsigned)sizeof(T));
+      xo[s] = one[0];
+      const long roff = (long)(r < 0 ? 0 : r) * a.M;
+#pragma unroll
+      for (int g = 0; g < NG; g++) {
+        const vec_t v = *reinterpret_cast<const vec_t *>(wcol[g] + roff);
+#pragma unroll
+        for (int c2 = 0; c2 < VW; c2++) wo[s][g][c2] = v[c2];
+      }
+    }
+  };
+  auto compute = [&](const T(&xi)[VW], const T(&wi)[VW][NG][VW]) {
+#pragma unroll
+    for (int s = 0; s < VW; s++)
+#pragma unroll
+      for (int g = 0; g < NG; g++)
+#pragma unroll
+        for (int c = 0; c < VW; c++) acc[g][c] = Real<T>::mfma(xi[s], wi[s][g][c], acc[g][c]);
+  };
+
+  for (long seg0 = 0;;) {
+    publish_segment(seg0);
+    __syncthreads();
+    request(w, xr[0], wr[0]);  // this wavefront's first chunk of the segment
+    SB_PHASE_MARK(12);
+    // chunks w, w + NWAVES, ... of the segment that hold list entries: n of them (at least 1 in the
+    // first segment, see above)
+    const long left = (long)cnt - seg0;  // entries from the start of this segment
+    const long segc = left >= SEG ? SEGC : (left + KC - 1) / KC;
+    long n = w < segc ? (segc - 1 - w) / NWAVES + 1 : 0;
+    if (seg0 == 0 && n == 0) n = 1;
+    const bool more = left > SEG;
+    if (more) request_segment(seg0 + SEG);  // uniform
+    __builtin_amdgcn_sched_barrier(0);
+    long i = 0;
+    for (; i + 2 <= n; i += 2) {
+      // the scheduling fences keep the requests where they are written, ahead of the MFMAs
+      request(w + (int)(i + 1) * NWAVES, xr[1], wr[1]);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(xr[0], wr[0]);
+      __builtin_amdgcn_sched_barrier(0);
+      request(w + (int)(i + 2) * NWAVES, xr[0], wr[0]);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(xr[1], wr[1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (i < n) compute(xr[0], wr[0]);
+    if (!more) break;
+    seg0 += SEG;
+    __syncthreads();  // everyone is done with the staged segment
+  }
+  SB_PHASE_MARK(1);
+  forward_finish<T, NG, true, NWAVES, VW>(acc, bv, red, a.act, a.B, a.M, b0, j0, ncol);
+  SB_PHASE_MARK(3);
+}
+
+}  // namespace sb

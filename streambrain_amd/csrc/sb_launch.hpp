@@ -31,7 +31,7 @@ struct TraceScalars {
 // with a pair of HIP events on the launch stream; sb_profile_stop sums the elapsed times per kernel.
 enum KernelId {
   K_FORWARD = 0, K_SOFTMAX, K_UPDATE_BIAS, K_UPDATE_BIAS_REG, K_MASK_SCORES,
-  K_MASK_SWAP, K_MASK_FIX, K_APPLY_MASK, K_ARGMAX, K_GATHER, K_FILL, K_TRAIN_FUSED, K_COUNT
+  K_MASK_SWAP, K_MASK_FIX, K_APPLY_MASK, K_ARGMAX, K_GATHER, K_FILL, K_TRAIN_FUSED, K_MASK_ROWS, K_COUNT
 };
 const char *kernel_name(int id);
 struct ProfScope {
@@ -61,6 +61,17 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
 template <typename T>
 int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias, long B, long N,
                    long H, long Mc, bool softmax);
+// The same result for a layer whose W is zero wherever wmask is 0, from the per-hypercolumn lists of
+// connected rows that launch_mask_rows builds (rows: [H, cap] ascending indices, the rest -1; cap a
+// multiple of 16; row_cnt: [H]); forward_rows_supported says whether the kernel takes the shape.
+template <typename T>
+bool forward_rows_supported(const T *W, long N, long H, long Mc);
+template <typename T>
+int launch_forward_rows(hipStream_t st, T *act, const T *x, const T *W, const T *bias, const int *rows,
+                        const int *row_cnt, long cap, long B, long N, long H, long Mc);
+// Lists of hypercolumns h0 .. h0 + count - 1 rebuilt from wmask.
+int launch_mask_rows(hipStream_t st, int *rows, int *row_cnt, const uint8_t *wmask, long N, long H,
+                     long cap, long h0, long count);
 template <typename T>
 int launch_softmax(hipStream_t st, T *act, long B, long H, long Mc);
 // Fused Ci/Cj/Cij + weights (+ regularised bias when bias_mode == 1, + mask when wmask != nullptr).

@@ -3,6 +3,7 @@
 #pragma once
 #include "sb_kernels.hpp"
 #include "sb_k_train.hpp"
+#include "sb_k_forward_rows.hpp"
 #include "sb_k_skinny.hpp"
 #include "sb_launch.hpp"
 
@@ -97,6 +98,42 @@ int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias
   if (rc) return rc;
   if (softmax) return launch_softmax<T>(st, act, B, H, Mc);
   return 0;
+}
+
+// ------------------------------------------------------------------- forward over the connected rows
+template <typename T>
+bool forward_rows_supported(const T *W, long N, long H, long Mc) {
+  constexpr int VW = Real<T>::VW;
+  const long M = H * Mc;
+  return M > 32 && M % VW == 0 && Mc % VW == 0 && aligned16(W) &&
+         cdiv(Mc, 16 * VW) <= (sizeof(T) == 4 ? 4 : 7) && 16 * N * (long)sizeof(T) < (1L << 31);
+}
+
+template <typename T, int NG>
+static int forward_rows_variant(hipStream_t st, const ForwardRowsArgs<T> &a) {
+  ProfScope prof_(st, K_FORWARD);
+  const long grid = 8 * cdiv(a.f.col_tiles * a.f.batch_tiles, 8);
+  SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
+  hipLaunchKernelGGL((k_forward_rows<T, NG, 8>), dim3((unsigned)grid), dim3(512), 0, st, a);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
+int launch_forward_rows(hipStream_t st, T *act, const T *x, const T *W, const T *bias, const int *rows,
+                        const int *row_cnt, long cap, long B, long N, long H, long Mc) {
+  SB_REQUIRE(act && x && W && bias && rows && row_cnt, "null pointer");
+  SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");
+  SB_REQUIRE(H * Mc < (1L << 31) && N < (1L << 31), "dimension too large");
+  SB_REQUIRE(cap > 0 && cap % 16 == 0, "row lists must be padded to a multiple of 16");
+  SB_REQUIRE(forward_rows_supported<T>(W, N, H, Mc), "shape not supported by the row-list forward kernel");
+  ForwardRowsArgs<T> a{{act, x, W, bias, B, N, H * Mc, Mc, H, cdiv(B, 16)}, rows, row_cnt, cap};
+  const long need = cdiv(Mc, 16 * Real<T>::VW);
+  if (need <= 1) return forward_rows_variant<T, 1>(st, a);
+  if (need <= 2) return forward_rows_variant<T, 2>(st, a);
+  if (need <= 4) return forward_rows_variant<T, 4>(st, a);
+  if constexpr (sizeof(T) == 8) return forward_rows_variant<T, 7>(st, a);
+  return -1;
 }
 
 template <typename T>
@@ -288,6 +325,9 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
 #define SB_INSTANTIATE_LAUNCHERS(T)                                                                   \
   template int launch_forward<T>(hipStream_t, T *, const T *, const T *, const T *, long, long, long, \
                                  long, bool);                                                         \
+  template bool forward_rows_supported<T>(const T *, long, long, long);                               \
+  template int launch_forward_rows<T>(hipStream_t, T *, const T *, const T *, const T *, const int *, \
+                                      const int *, long, long, long, long, long);                     \
   template int launch_softmax<T>(hipStream_t, T *, long, long, long);                                 \
   template int launch_train_fused<T>(hipStream_t, const T *, const T *, T *, T *, const T *, const T *, \
                                      T *, T *, const uint8_t *, int, T *, T *, long, long, long, long, \

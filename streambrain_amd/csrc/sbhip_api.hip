@@ -55,7 +55,7 @@ const char *kernel_name(int id) {
   static const char *names[K_COUNT] = {"forward", "softmax", "update_bias",
                                        "update_bias_regularized", "mask_scores", "mask_swap",
                                        "mask_fix_weights", "apply_mask", "argmax", "gather_rows", "fill",
-                                       "train_fused"};
+                                       "train_fused", "mask_rows"};
   return (id >= 0 && id < K_COUNT) ? names[id] : "?";
 }
 
@@ -153,6 +153,13 @@ struct Layer {
   long act_rows = 0;
   void *nom = nullptr;  // rewiring scratch [N]
   int *csum = nullptr;
+  // Sparse layers (at most half of wmask set): per-hypercolumn lists of the connected rows for the
+  // forward pass, kept in step with wmask.  They are used while W is known to be zero wherever wmask
+  // is 0, which a training step establishes and a write to W or wmask through the state interface
+  // ends.
+  int *rows = nullptr, *row_cnt = nullptr;
+  long rows_cap = 0;
+  bool w_masked = false;
 };
 
 }  // namespace sb
@@ -212,7 +219,9 @@ static int layer_free(Layer &L) {
   rc |= free_dev(L.W); rc |= free_dev(L.bias); rc |= free_dev(L.Ci); rc |= free_dev(L.Cj);
   rc |= free_dev(L.Cij); rc |= free_dev(L.kbi); rc |= free_dev(w); rc |= free_dev(L.act);
   rc |= free_dev(L.nom); rc |= free_dev(c); rc |= free_dev(L.Ci_alt); rc |= free_dev(L.Cj_alt);
-  L.wmask = nullptr; L.csum = nullptr;
+  void *r = L.rows, *rc_ = L.row_cnt;
+  rc |= free_dev(r); rc |= free_dev(rc_);
+  L.wmask = nullptr; L.csum = nullptr; L.rows = nullptr; L.row_cnt = nullptr; L.rows_cap = 0;
   return rc;
 }
 
@@ -230,6 +239,9 @@ static int ensure_act(sb_net *net, long rows) {
 
 template <typename T>
 static int layer_forward(const Layer &L, const T *x, long B) {
+  if (L.rows && L.w_masked)
+    return launch_forward_rows<T>(g_ctx.stream, (T *)L.act, x, (const T *)L.W, (const T *)L.bias, L.rows,
+                                  L.row_cnt, L.rows_cap, B, L.N, L.H, L.Mc);
   return launch_forward<T>(g_ctx.stream, (T *)L.act, x, (const T *)L.W, (const T *)L.bias, B, L.N, L.H,
                            L.Mc, true);
 }
@@ -250,6 +262,7 @@ static int layer_train_step(Layer &L, const T *x, const T *y, long B, long h) {
   if (rc) return rc;
   std::swap(L.Ci, L.Ci_alt);
   std::swap(L.Cj, L.Cj_alt);
+  if (L.plastic) L.w_masked = true;  // every entry of W has just been written under the mask
   if (L.plastic && h >= 0) {
     rc = launch_update_mask<T>(st, L.wmask, (const T *)nullptr, (const T *)L.Ci, (const T *)L.Cj,
                                (const T *)L.Cij, cthr, L.N, L.H, L.Mc, h, 16, (T *)L.nom, L.csum);
@@ -257,8 +270,40 @@ static int layer_train_step(Layer &L, const T *x, const T *y, long B, long h) {
     rc = launch_mask_fix_weights<T>(st, (T *)L.W, L.wmask, (const T *)L.Ci, (const T *)L.Cj,
                                     (const T *)L.Cij, cthr, L.N, L.H, L.Mc, h);
     if (rc) return rc;
+    // a swap leaves the number of connected rows of the hypercolumn as it was, so the list fits
+    if (L.rows) rc = launch_mask_rows(st, L.rows, L.row_cnt, L.wmask, L.N, L.H, L.rows_cap, h, 1);
+    if (rc) return rc;
   }
   return 0;
+}
+
+// After wmask has been replaced from the host copy `mask` [N, H]: (re)build the row lists when at most
+// half of the connections exist and the forward kernel over row lists takes the layer's shape, drop
+// them otherwise.
+template <typename T>
+static int layer_mask_replaced(Layer &L, const uint8_t *mask) {
+  L.w_masked = false;
+  std::vector<long> count((size_t)L.H, 0);
+  for (long i = 0; i < L.N; i++)
+    for (long h = 0; h < L.H; h++) count[(size_t)h] += mask[i * L.H + h] != 0;
+  long total = 0, most = 0;
+  for (long c : count) total += c, most = c > most ? c : most;
+  const bool sparse = 2 * total <= L.N * L.H && forward_rows_supported<T>((const T *)L.W, L.N, L.H, L.Mc);
+  const long cap = (most + 15) / 16 * 16 + 16;
+  if (!sparse || cap > L.rows_cap) {
+    SB_HIP(hipStreamSynchronize(g_ctx.stream));
+    void *r = L.rows, *c = L.row_cnt;
+    int rc = free_dev(r) | free_dev(c);
+    L.rows = nullptr; L.row_cnt = nullptr; L.rows_cap = 0;
+    if (rc) return rc;
+  }
+  if (!sparse) return 0;
+  if (!L.rows) {
+    SB_HIP(hipMalloc((void **)&L.rows, (size_t)L.H * cap * sizeof(int)));
+    SB_HIP(hipMalloc((void **)&L.row_cnt, (size_t)L.H * sizeof(int)));
+    L.rows_cap = cap;
+  }
+  return launch_mask_rows(g_ctx.stream, L.rows, L.row_cnt, L.wmask, L.N, L.H, L.rows_cap, 0, L.H);
 }
 
 template <typename T>
@@ -517,6 +562,10 @@ int sb_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes) {
   SB_HIP(hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, g_ctx.stream));
   return 0;
 }
+int sb_mask_rows(int *d_rows, int *d_row_cnt, const uint8_t *d_wmask, long N, long H, long cap) {
+  SB_READY();
+  return launch_mask_rows(g_ctx.stream, d_rows, d_row_cnt, d_wmask, N, H, cap, 0, H);
+}
 int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
   SB_READY();
   return launch_fill_bytes(g_ctx.stream, d_dst, value, bytes);
@@ -537,6 +586,11 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
     SB_READY();                                                                                        \
     SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");                           \
     return launch_forward<T>(g_ctx.stream, act, x, W, bias, B, N, H, Mc, true);                        \
+  }                                                                                                    \
+  int sb_compute_activation_rows_##SFX(T *act, const T *x, const T *W, const T *bias, const int *rows, \
+                                       const int *row_cnt, long cap, long B, long N, long H, long Mc) { \
+    SB_READY();                                                                                        \
+    return launch_forward_rows<T>(g_ctx.stream, act, x, W, bias, rows, row_cnt, cap, B, N, H, Mc);     \
   }                                                                                                    \
   int sb_update_weights_##SFX(T *Ci, T *Cj, T *Cij, const T *a_i, const T *a_o, T taupdt, T *W,        \
                               T cthr, long B, long N, long M) {                                        \
@@ -678,7 +732,14 @@ int sb_net_set_layer_state(sb_net *net, int layer, const char *name, const void 
   if (rc) return rc;
   SB_REQUIRE(h_src, "null pointer");
   SB_REQUIRE(bytes == s.bytes, "size mismatch");
-  return sb_memcpy_h2d(s.ptr, h_src, bytes);
+  rc = sb_memcpy_h2d(s.ptr, h_src, bytes);
+  if (rc) return rc;
+  Layer &L = net->layers[layer];
+  if (s.ptr == L.W) L.w_masked = false;
+  if (s.ptr == L.wmask)
+    return net->dtype == SB_F32 ? layer_mask_replaced<float>(L, (const uint8_t *)h_src)
+                                : layer_mask_replaced<double>(L, (const uint8_t *)h_src);
+  return 0;
 }
 
 int sb_net_get_layer_state(sb_net *net, int layer, const char *name, void *h_dst, size_t bytes) {

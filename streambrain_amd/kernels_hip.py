@@ -61,6 +61,34 @@ def compute_activation(weights, bias, inputs, hypercolumns, minicolumns):
     return d_act.numpy()
 
 
+def mask_rows(wmask):
+    """Per-hypercolumn lists of the connected rows of wmask[N, H]: (rows[H, cap], counts[H]); rows holds
+    ascending indices, then -1 up to cap."""
+    wmask = np.ascontiguousarray(wmask, dtype=np.uint8)
+    N, H = wmask.shape
+    cap = (int(np.count_nonzero(wmask, axis=0).max(initial=0)) + 15) // 16 * 16 + 16
+    d_rows = _dev(np.full((H, cap), -2, dtype=np.int32))
+    d_cnt = DeviceArray((H,), np.int32)
+    check(lib().sb_mask_rows(d_rows.ptr, d_cnt.ptr, _dev(wmask).ptr, N, H, cap))
+    return d_rows.numpy(), d_cnt.numpy()
+
+
+def compute_activation_rows(weights, bias, inputs, wmask, hypercolumns, minicolumns):
+    """compute_activation for weights that are zero wherever wmask is 0, over the connected rows only."""
+    dt = weights.dtype
+    f = _fn("sb_compute_activation_rows", dt)
+    B, N = inputs.shape
+    M = hypercolumns * minicolumns
+    assert weights.shape == (N, M) and bias.shape == (M,) and wmask.shape == (N, hypercolumns)
+    rows, cnt = mask_rows(wmask)
+    d_act = DeviceArray((B, M), dt)
+    d_x, d_w, d_b = _dev(inputs, dt), _dev(weights, dt), _dev(bias, dt)
+    d_rows, d_cnt = _dev(rows), _dev(cnt)
+    check(f(d_act.ptr, d_x.ptr, d_w.ptr, d_b.ptr, d_rows.ptr, d_cnt.ptr, rows.shape[1], B, N,
+            hypercolumns, minicolumns))
+    return d_act.numpy()
+
+
 def update_weights(Ci, Cj, Cij, a_i, a_o, taupdt, weights, cthr):
     dt = Ci.dtype
     f = _fn("sb_update_weights", dt)

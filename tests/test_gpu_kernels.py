@@ -50,6 +50,50 @@ def test_update_state(k, oracle, dtype, B, N, M):
     assert_close(ref, exact, dtype, "oracle vs exact", scale)
 
 
+# ------------------------------------------------------------- forward over the connected rows only
+@pytest.mark.parametrize("N,H,density", [(1, 1, 1.0), (40, 3, 0.3), (1568, 30, 0.1), (300, 5, 0.0),
+                                         (257, 4, 0.05), (64, 2, 1.0)])
+def test_mask_rows(k, N, H, density):
+    rng = np.random.default_rng(N + H)
+    wmask = (rng.random((N, H)) < density).astype(np.uint8)
+    if N > 100:
+        wmask[:, 1] = 0  # an unconnected hypercolumn
+    rows, cnt = k.mask_rows(wmask)
+    for h in range(H):
+        want = np.flatnonzero(wmask[:, h])
+        assert cnt[h] == want.size
+        assert np.array_equal(rows[h, :want.size], want)
+        assert np.all(rows[h, want.size:] == -1)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("B,N,H,Mc,density", [(128, 1568, 30, 100, 0.1), (96, 1568, 30, 100, 0.1),
+                                              (7, 40, 3, 12, 0.3), (33, 300, 2, 200, 0.2),
+                                              (16, 64, 2, 64, 1.0), (20, 100, 2, 256, 0.05),
+                                              (5, 50, 3, 12, 0.0), (300, 5000, 4, 100, 0.4),
+                                              (12, 40, 2, 224, 0.5)])
+def test_compute_activation_rows(k, oracle, dtype, B, N, H, Mc, density):
+    """The row-list forward kernel against the dense reference computation on the masked weights."""
+    if dtype == np.float32 and Mc % 4:
+        pytest.skip("float32 needs minicolumns divisible by 4")
+    if dtype == np.float64 and Mc > 224:
+        pytest.skip("float64 takes hypercolumns of at most 224 minicolumns")
+    rng = np.random.default_rng(B + N + H + Mc)
+    M = H * Mc
+    wmask = (rng.random((N, H)) < density).astype(np.uint8)
+    x = rng.random((B, N)).astype(dtype)
+    W = (0.1 * rng.standard_normal((N, M))).astype(dtype) * np.repeat(wmask, Mc, axis=1).astype(dtype)
+    b = (0.1 * rng.random(M)).astype(dtype)
+    got = k.compute_activation_rows(W, b, x, wmask, H, Mc)
+    ref = oracle.update_state(np.zeros((B, M), dtype=dtype), W, b, x)
+    ref = oracle.softmax_minicolumns(ref, H, Mc)
+    scale = max(1.0, np.sqrt(N / 64.0)) if dtype == np.float32 else 4.0
+    assert_close(got, ref, dtype, "gpu vs oracle", scale)
+    assert np.allclose(got.reshape(B, H, Mc).sum(2), 1.0, atol=100 * TOL[dtype])
+    # and the dense kernel on the same operands
+    assert_close(got, k.compute_activation(W, b, x, H, Mc), dtype, "rows vs dense", scale)
+
+
 # ----------------------------------------------------------------------------------------- softmax
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("B,H,Mc", [(1, 1, 1), (5, 3, 7), (128, 30, 100), (9, 2, 300), (4, 1, 10)])
