@@ -171,6 +171,9 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
     __syncthreads();
     request(w, xr[0], wr[0]);  // this wavefront's first chunk of the segment
     SB_PHASE_MARK(12);
+#ifdef SB_PHASE_WAIT
+    SB_PHASE_WAIT();
+#endif
     // chunks w, w + NWAVES, ... of the segment that hold list entries: n of them (at least 1 in the
     // first segment, see above)
     const long left = (long)cnt - seg0;  // entries from the start of this segment

@@ -51,6 +51,7 @@ struct TrainArgs {
   T *Ci_next;    // new traces (written by the first tile column / row)
   T *Cj_next;
   const uint8_t *wmask;  // [N,H] or nullptr (no mask: every synapse active)
+  int w_masked;          // W is already zero wherever wmask is 0: such entries need not be written
   int bias_mode;         // 0: leave bias alone; 1: update_bias_regularized on the new Cj
   T *bias, *kbi;
   long B, N, M, H, Mc;
@@ -289,17 +290,26 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
     const int lr = er + RPP * k;  // rows past the matrix compute garbage that the window drops
     const T rci = rci_s[lr];
     const bool row_live = !(rci < T(0)) && (MB != 1 || !masked || mb[k][0] != 0);
-    T cv[VW], wv[VW];
+    T cv[VW];
 #pragma unroll
     for (int e = 0; e < VW; e++) {
-      T cn = cpre[k][e] * a.omt + cs[lr * CP + VW * eg + e] * scale;
-      cn = fmax(cn, T(0));  // 0 as well when cn is NaN, like the reference's `cn > 0 ? cn : 0`
-      cv[e] = cn;
-      const T wgt = R::wlog(fmax(cn, a.cthr4) * rci * rcj[e]);
+      const T cn = cpre[k][e] * a.omt + cs[lr * CP + VW * eg + e] * scale;
+      cv[e] = fmax(cn, T(0));  // 0 as well when cn is NaN, like the reference's `cn > 0 ? cn : 0`
+    }
+    cwin.template store<VEC>(cv, tat, k * pass_bytes, ecol, a.M);
+    // Where the mask is 0 the weight is 0, and when the caller vouches that W holds 0 there already, a
+    // wavefront whose vectors all lie under zero mask bytes has nothing to compute or store.
+    bool connected = !masked;
+#pragma unroll
+    for (int e = 0; e < MB; e++) connected = connected || mb[k][e] != 0;
+    if (a.w_masked && __builtin_amdgcn_ballot_w64(connected) == 0) continue;
+    T wv[VW];
+#pragma unroll
+    for (int e = 0; e < VW; e++) {
+      const T wgt = R::wlog(fmax(cv[e], a.cthr4) * rci * rcj[e]);
       const bool keep = row_live && col_live[e] && (MB == 1 || !masked || mb[k][e] != 0);
       wv[e] = keep ? wgt : T(0);
     }
-    cwin.template store<VEC>(cv, tat, k * pass_bytes, ecol, a.M);
     wwin.template store<VEC>(wv, tat, k * pass_bytes, ecol, a.M);
   }
   SB_PHASE_MARK(14);

@@ -153,7 +153,8 @@ int launch_softmax(hipStream_t st, T *act, long B, long H, long Mc) {
 template <typename T>
 int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci, const T *Cj,
                        T *Ci_next, T *Cj_next, const uint8_t *wmask, int bias_mode, T *bias, T *kbi,
-                       long B, long N, long H, long Mc, T taupdt, T cthr, T khalf, T pmin, T taubdt) {
+                       long B, long N, long H, long Mc, T taupdt, T cthr, T khalf, T pmin, T taubdt,
+                       bool w_masked) {
   constexpr int VW = Real<T>::VW;
   SB_REQUIRE(x && y && Cij && W && Ci && Cj && Ci_next && Cj_next, "null pointer");
   SB_REQUIRE(Ci != Ci_next && Cj != Cj_next, "old and new traces must be distinct buffers");
@@ -164,7 +165,7 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   const TraceScalars<T> s = TraceScalars<T>::from(taupdt, cthr);
   TrainArgs<T> a;
   a.x = x; a.y = y; a.Cij = Cij; a.W = W; a.Ci = Ci; a.Cj = Cj; a.Ci_next = Ci_next; a.Cj_next = Cj_next;
-  a.wmask = wmask; a.bias_mode = bias_mode; a.bias = bias; a.kbi = kbi;
+  a.wmask = wmask; a.w_masked = (wmask && w_masked) ? 1 : 0; a.bias_mode = bias_mode; a.bias = bias; a.kbi = kbi;
   a.B = B; a.N = N; a.M = M; a.H = H; a.Mc = Mc;
   a.tau = s.tau; a.omt = s.omt; a.fB = (T)B; a.invB = (T)1 / (T)B; a.cthr = s.cthr; a.cthr4 = s.cthr4;
   a.khalf = khalf; a.pmin = pmin; a.taubdt = taubdt;
@@ -331,7 +332,7 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
   template int launch_softmax<T>(hipStream_t, T *, long, long, long);                                 \
   template int launch_train_fused<T>(hipStream_t, const T *, const T *, T *, T *, const T *, const T *, \
                                      T *, T *, const uint8_t *, int, T *, T *, long, long, long, long, \
-                                     T, T, T, T, T);                                                   \
+                                     T, T, T, T, T, bool);                                             \
   template int launch_update_bias<T>(hipStream_t, T *, const T *, T, long);                           \
   template int launch_update_bias_regularized<T>(hipStream_t, T *, T *, const T *, T, T, T, T, long); \
   template int launch_update_mask<T>(hipStream_t, uint8_t *, const T *, const T *, const T *,         \

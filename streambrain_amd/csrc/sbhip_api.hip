@@ -134,7 +134,7 @@ static int train_in_place(const T *x, const T *y, T *Cij, T *W, T *Ci, T *Cj, co
   if (rc) return rc;
   T *ci_next = (T *)g_ctx.trace_next, *cj_next = ci_next + N;
   rc = launch_train_fused<T>(st, x, y, Cij, W, Ci, Cj, ci_next, cj_next, wmask, bias_mode, bias, kbi, B,
-                             N, H, Mc, taupdt, cthr, khalf, pmin, taubdt);
+                             N, H, Mc, taupdt, cthr, khalf, pmin, taubdt, false);
   if (rc) return rc;
   SB_HIP(hipMemcpyAsync(Ci, ci_next, (size_t)N * sizeof(T), hipMemcpyDeviceToDevice, st));
   SB_HIP(hipMemcpyAsync(Cj, cj_next, (size_t)M * sizeof(T), hipMemcpyDeviceToDevice, st));
@@ -258,7 +258,7 @@ static int layer_train_step(Layer &L, const T *x, const T *y, long B, long h) {
   rc = launch_train_fused<T>(st, x, y, (T *)L.Cij, (T *)L.W, (const T *)L.Ci, (const T *)L.Cj,
                              (T *)L.Ci_alt, (T *)L.Cj_alt, L.plastic ? L.wmask : nullptr,
                              L.plastic ? 1 : 0, (T *)L.bias, (T *)L.kbi, B, L.N, L.H, L.Mc, tau, cthr,
-                             (T)L.khalf, (T)L.pmin, (T)L.taubdt);
+                             (T)L.khalf, (T)L.pmin, (T)L.taubdt, L.w_masked);
   if (rc) return rc;
   std::swap(L.Ci, L.Ci_alt);
   std::swap(L.Cj, L.Cj_alt);
