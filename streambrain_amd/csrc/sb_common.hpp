@@ -166,11 +166,9 @@ struct BufferWindow {
   static constexpr unsigned kOutside = 0x80000000u;  // beyond any window, also after adding a uniform offset
   __amdgpu_buffer_rsrc_t rsrc;
   __device__ BufferWindow(const T *base, long elems) {
-    // window size = clamp(elems * sizeof(T), 0, 2 GiB), written so that it stays on the scalar unit when
-    // `elems` is uniform (a 64-bit signed compare would go to the vector unit)
-    const unsigned long bytes = (unsigned long)elems * sizeof(T);
-    const unsigned hi = (unsigned)(bytes >> 31);  // 0 for 0 <= bytes < 2 GiB; negative sizes have bit 32 set
-    const unsigned size = hi == 0 ? (unsigned)bytes : (((unsigned)(bytes >> 63)) ? 0u : 0x80000000u);
+    // window size = clamp(elems * sizeof(T), 0, 2 GiB)
+    const long bytes = elems > 0 ? elems * (long)sizeof(T) : 0;
+    const unsigned size = (unsigned)(bytes < 0x80000000L ? bytes : 0x80000000L);
     // descriptor word 3 = 0x00020000: raw buffer, 32-bit data format, as for every untyped gfx9 buffer
     rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(base), 0, (int)size, 0x00020000);
   }

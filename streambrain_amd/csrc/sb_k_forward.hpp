@@ -156,9 +156,9 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
   }
 }
 
-// Unguarded 16-byte loads of the main loop: rows / columns outside the matrix are redirected to a valid
-// address (their products land in accumulator rows / columns that are never stored), so the loop body
-// is loads + MFMAs + pointer bumps only.  The last, partial K chunk takes the guarded path.
+// Main loop: x and W are read with 16-byte loads through bounds-checked buffer windows, so rows and
+// columns outside the matrices read zero and the loop body is loads + MFMAs only.  The last, partial K
+// chunk (and shapes without 16-byte alignment) take the guarded path.
 // One workgroup per CU is all the tiling provides at small batch sizes, so the register allocator is told
 // to aim for NWAVES/4 wavefronts per SIMD and spend the registers on loads in flight instead.
 //
