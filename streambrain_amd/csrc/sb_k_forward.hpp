@@ -51,18 +51,37 @@ struct PackedCols {  // LW consecutive elements, element-aligned
   T v[LW];
 } __attribute__((packed, aligned(sizeof(T))));
 
+// The epilogue's split of a tile row over threads: all 64*NWAVES threads take part, TPR of them per batch
+// row (a power of two, at most 64, so a row never straddles wavefronts), each with PT columns
+// lr + TPR t.  load() fetches the thread's bias values; the kernels call it ahead of their main loop so
+// that the latency is not added to the epilogue.
+template <typename T, int NG, int NWAVES>
+struct ForwardBias {
+  static constexpr int TPR = 4 * NWAVES;
+  static constexpr int COLS = NG * 16 * Real<T>::VW;
+  static constexpr int PT = (COLS + TPR - 1) / TPR;
+  static_assert(TPR <= 64, "a batch row's threads must lie in one wavefront");
+  __device__ static __forceinline__ void load(T (&bv)[PT], const T *bias, long j0, long ncol) {
+    const int lr = threadIdx.x % TPR;
+#pragma unroll
+    for (int t = 0; t < PT; t++) {
+      const long col = lr + TPR * t;
+      bv[t] = bias[j0 + (col < ncol ? col : 0)];
+    }
+  }
+};
+
 // Tail of the forward kernels: the NWAVES partial tiles (one per wavefront, in MFMA accumulator layout)
 // are summed through LDS in a fixed order (deterministic), then 16 threads per batch row add the bias
-// and, when FUSE, do the softmax over the tile's ncol columns.  bv: the bias values of thread tid < 256
-// (columns tid % 16 + 16 t), loaded by the caller ahead of its main loop.
+// and, when FUSE, do the softmax over the tile's ncol columns.  bv: the thread's bias values
+// (ForwardBias::load).
 template <typename T, int NG, bool FUSE, int NWAVES, int LW>
 __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&acc)[NG][Real<T>::VW],
-                                               const T (&bv)[NG * Real<T>::VW],
+                                               const T (&bv)[ForwardBias<T, NG, NWAVES>::PT],
                                                T (&red)[NWAVES / 2][16][TileCols<T, NG, LW>::CP], T *act,
                                                long B, long M, long b0, long j0, long ncol) {
   using TC = TileCols<T, NG, LW>;
   constexpr int VW = Real<T>::VW;
-  constexpr int PER = NG * VW;
   using vec_t = typename Real<T>::vec_t;
   auto gwidth = [](int g) { return TC::gwidth(g); };
   auto gcol = [](int g, int p_) { return TC::gcol(g, p_); };
@@ -112,14 +131,14 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
   __syncthreads();
 
   SB_PHASE_MARK(2);
-  // ---- bias (+ softmax): 16 threads per batch row (256 threads), thread handles columns l16 + 16 t
-  if (tid >= 256) return;
-  const int row = tid >> 4, l16 = tid & 15;
-  T vals[PER];
+  // ---- bias (+ softmax): TPR threads per batch row, thread handles columns lr + TPR t
+  constexpr int TPR = ForwardBias<T, NG, NWAVES>::TPR, PT = ForwardBias<T, NG, NWAVES>::PT;
+  const int row = tid / TPR, lr = tid % TPR;
+  T vals[PT];
   T mx = -INFINITY;
 #pragma unroll
-  for (int t = 0; t < PER; t++) {
-    const long col = l16 + 16 * t;
+  for (int t = 0; t < PT; t++) {
+    const long col = lr + TPR * t;
     T sum = red[0][row][col < ncol ? col : 0];
 #pragma unroll
     for (int h = 1; h < HALF; h++) sum += red[h][row][col < ncol ? col : 0];
@@ -128,29 +147,29 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
   }
   if (FUSE) {
 #pragma unroll
-    for (int o = 8; o >= 1; o >>= 1) {
+    for (int o = TPR / 2; o >= 1; o >>= 1) {
       const T other = __shfl_xor(mx, o);
       mx = other > mx ? other : mx;
     }
     T sum = T(0);
 #pragma unroll
-    for (int t = 0; t < PER; t++) {
-      const long col = l16 + 16 * t;
+    for (int t = 0; t < PT; t++) {
+      const long col = lr + TPR * t;
       if (col < ncol) {
         vals[t] = Real<T>::exp_(vals[t] - mx);
         sum += vals[t];
       }
     }
 #pragma unroll
-    for (int o = 8; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+    for (int o = TPR / 2; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
 #pragma unroll
-    for (int t = 0; t < PER; t++) vals[t] = vals[t] / sum;
+    for (int t = 0; t < PT; t++) vals[t] = vals[t] / sum;
   }
   if (b0 + row < B) {
     T *out = act + (b0 + row) * M + j0;
 #pragma unroll
-    for (int t = 0; t < PER; t++) {
-      const long col = l16 + 16 * t;
+    for (int t = 0; t < PT; t++) {
+      const long col = lr + TPR * t;
       if (col < ncol) out[col] = vals[t];
     }
   }
@@ -237,16 +256,10 @@ void k_forward(ForwardArgs<T> a) {
     }
   };
 
-  // the epilogue's bias values (thread tid < 256: batch row tid / 16, columns tid % 16 + 16 t) are
-  // requested before the K loop, so their latency is not added to the epilogue
-  constexpr int PER = NG * VW;
+  // the epilogue's bias values are requested before the K loop, so their latency is not added to it
   const long ncol = jend - j0;
-  T bv[PER];
-#pragma unroll
-  for (int t = 0; t < PER; t++) {
-    const long col = (tid & 15) + 16 * t;
-    bv[t] = a.bias[j0 + (col < ncol ? col : 0)];
-  }
+  T bv[ForwardBias<T, NG, NWAVES>::PT];
+  ForwardBias<T, NG, NWAVES>::load(bv, a.bias, j0, ncol);
   const long nfull = a.N / KC;  // chunks with all KC reduction indices inside the matrix
   SB_PHASE_MARK(0);
   if (VEC) {

@@ -119,13 +119,8 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
 #pragma unroll
     for (int c = 0; c < VW; c++) acc[g][c] = acc_t{0, 0, 0, 0};
 
-  constexpr int PER = NG * VW;
-  T bv[PER];
-#pragma unroll
-  for (int t = 0; t < PER; t++) {
-    const long col = (tid & 15) + 16 * t;
-    bv[t] = a.bias[j0 + (col < ncol ? col : 0)];
-  }
+  T bv[ForwardBias<T, NG, NWAVES>::PT];
+  ForwardBias<T, NG, NWAVES>::load(bv, a.bias, j0, ncol);
 
   // x through a bounds-checked window over this tile's 16 batch rows: rows past the batch and padding
   // entries (offset kOutside) read zero
