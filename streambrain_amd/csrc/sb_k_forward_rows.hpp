@@ -63,7 +63,8 @@ struct ForwardRowsArgs {
 // segment, which is padding where the list is shorter.
 // Requires M % VW == 0, Mc % VW == 0 and 16-byte aligned W.
 template <typename T, int NG, int NWAVES>
-__global__ __launch_bounds__(64 * NWAVES) __attribute__((amdgpu_waves_per_eu(NWAVES / 4, NWAVES / 4)))
+__global__ __launch_bounds__(64 * NWAVES)
+__attribute__((amdgpu_waves_per_eu(NWAVES >= 4 ? NWAVES / 4 : 1, NWAVES >= 4 ? NWAVES / 4 : 1)))
 void k_forward_rows(ForwardRowsArgs<T> ar) {
   const ForwardArgs<T> &a = ar.f;
   constexpr int VW = Real<T>::VW;
