@@ -4,46 +4,13 @@
 // wherever wmask[i, h] is 0, so in  act = softmax_per_hypercolumn(x . W + bias)  (omp.cc:70-87 +
 // kernels_numpy.py:13-25) those rows add exact zeros to hypercolumn h.  With a connection density of
 // 0.1 nine tenths of the reduction are such zeros.  k_forward_rows skips them: per hypercolumn it walks
-// the ascending list of connected rows (k_mask_rows keeps the lists in step with wmask) and gathers
+// the ascending list of connected rows (k_mask_rows in sb_kernels.hpp keeps the lists in step with wmask) and gathers
 // those rows of W and those columns of x.  Same tiling, accumulator layout and epilogue as k_forward.
 #pragma once
 #include "sb_k_forward.hpp"
+#include "sb_kernels.hpp"
 
 namespace sb {
-
-// rows[h * cap + 0 .. cnt_h) = ascending indices i with wmask[i, h] != 0, the rest of the cap entries
-// -1; row_cnt[h] = cnt_h.  One workgroup per hypercolumn h0 + blockIdx.x; entries beyond
-// `cap` are dropped (the host sizes cap from the column counts, so none are).  (A template only so that
-// the header can be included from several translation units.)
-template <int = 0>
-__global__ __launch_bounds__(256) void k_mask_rows(int *rows, int *row_cnt, const uint8_t *wmask, long N,
-                                                   long H, long cap, long h0) {
-  __shared__ int scan[256];
-  const int tid = threadIdx.x;
-  const long h = h0 + blockIdx.x;
-  const long seg = (N + 255) / 256;
-  const long lo = tid * seg < N ? tid * seg : N, hi = lo + seg < N ? lo + seg : N;
-  int mine = 0;
-  for (long i = lo; i < hi; i++) mine += wmask[i * H + h] != 0;
-  scan[tid] = mine;
-  __syncthreads();
-  for (int o = 1; o < 256; o <<= 1) {  // inclusive scan of the per-thread counts
-    const int other = tid >= o ? scan[tid - o] : 0;
-    __syncthreads();
-    scan[tid] += other;
-    __syncthreads();
-  }
-  int *list = rows + h * cap;
-  long pos = scan[tid] - mine;
-  for (long i = lo; i < hi; i++)
-    if (wmask[i * H + h] != 0) {
-      if (pos < cap) list[pos] = (int)i;
-      pos++;
-    }
-  const long total = scan[255] < cap ? scan[255] : cap;
-  for (long k = total + tid; k < cap; k += 256) list[k] = -1;
-  if (tid == 0) row_cnt[h] = (int)total;
-}
 
 template <typename T>
 struct ForwardRowsArgs {

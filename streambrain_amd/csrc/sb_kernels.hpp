@@ -91,6 +91,7 @@ __global__ __launch_bounds__(256) void k_apply_mask(T *W, const uint8_t *wmask, 
 //   picked only when it belongs to the first candidate row.
 // Step 3 (k_mask_fix_weights): rewrites W[:, hypercolumn h] under the new mask (network path only,
 //   where W is kept masked).
+// Step 4: see mask_rows_block below.
 // =====================================================================================================
 template <typename T>
 struct MaskArgs {
@@ -233,10 +234,57 @@ __global__ __launch_bounds__(1024) void k_mask_swap(MaskArgs<T> a) {
   }
 }
 
+// Step 4 (mask_rows_block / k_mask_rows): the list of connected rows of a hypercolumn, which the forward
+//   pass over connected rows walks:  rows[h * cap + 0 .. cnt_h) = ascending indices i with
+//   wmask[i, h] != 0, the rest of the cap entries -1; row_cnt[h] = cnt_h.  One workgroup of 256 threads
+//   per hypercolumn; entries beyond `cap` are dropped (the host sizes cap from the column counts, so
+//   none are).
+__device__ __forceinline__ void mask_rows_block(int *rows, int *row_cnt, const uint8_t *wmask, long N, long H,
+                                                long cap, long h) {
+  __shared__ int scan[256];
+  const int tid = threadIdx.x;
+  const long seg = (N + 255) / 256;
+  const long lo = tid * seg < N ? tid * seg : N, hi = lo + seg < N ? lo + seg : N;
+  int mine = 0;
+  for (long i = lo; i < hi; i++) mine += wmask[i * H + h] != 0;
+  scan[tid] = mine;
+  __syncthreads();
+  for (int o = 1; o < 256; o <<= 1) {  // inclusive scan of the per-thread counts
+    const int other = tid >= o ? scan[tid - o] : 0;
+    __syncthreads();
+    scan[tid] += other;
+    __syncthreads();
+  }
+  int *list = rows + h * cap;
+  long pos = scan[tid] - mine;
+  for (long i = lo; i < hi; i++)
+    if (wmask[i * H + h] != 0) {
+      if (pos < cap) list[pos] = (int)i;
+      pos++;
+    }
+  const long total = scan[255] < cap ? scan[255] : cap;
+  for (long k = total + tid; k < cap; k += 256) list[k] = -1;
+  if (tid == 0) row_cnt[h] = (int)total;
+}
+// hypercolumns h0 .. h0 + gridDim.x - 1  (a template only so that the header can be included from several
+// translation units)
+template <int = 0>
+__global__ __launch_bounds__(256) void k_mask_rows(int *rows, int *row_cnt, const uint8_t *wmask, long N,
+                                                   long H, long cap, long h0) {
+  mask_rows_block(rows, row_cnt, wmask, N, H, cap, h0 + blockIdx.x);
+}
+
+// Step 3; with a row list (rows != nullptr) one extra workgroup, the last, does step 4 for hypercolumn h
+// in the same launch.
 template <typename T>
 __global__ __launch_bounds__(256) void k_mask_fix_weights(T *W, const uint8_t *wmask, const T *Ci,
                                                           const T *Cj, const T *Cij, T cthr, T cthr4,
-                                                          long N, long M, long H, long Mc, long h) {
+                                                          long N, long M, long H, long Mc, long h, int *rows,
+                                                          int *row_cnt, long cap) {
+  if (rows != nullptr && blockIdx.x == gridDim.x - 1) {  // uniform over the workgroup
+    mask_rows_block(rows, row_cnt, wmask, N, H, cap, h);
+    return;
+  }
   const long e = (long)blockIdx.x * 256 + threadIdx.x;
   if (e >= N * Mc) return;
   const long i = e / Mc;

@@ -92,9 +92,11 @@ template <typename T>
 int launch_update_mask(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, const T *Cj,
                        const T *Cij, T cthr, long N, long H, long Mc, long h, long iterations, T *nom,
                        int *csum);
+// rows != nullptr: the row list of hypercolumn h (see launch_mask_rows) is rebuilt in the same launch.
 template <typename T>
 int launch_mask_fix_weights(hipStream_t st, T *W, const uint8_t *wmask, const T *Ci, const T *Cj,
-                            const T *Cij, T cthr, long N, long H, long Mc, long h);
+                            const T *Cij, T cthr, long N, long H, long Mc, long h, int *rows, int *row_cnt,
+                            long cap);
 template <typename T>
 int launch_apply_mask(hipStream_t st, T *W, const uint8_t *wmask, long N, long H, long Mc);
 template <typename T>

@@ -264,13 +264,17 @@ int launch_update_mask(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, 
 
 template <typename T>
 int launch_mask_fix_weights(hipStream_t st, T *W, const uint8_t *wmask, const T *Ci, const T *Cj,
-                            const T *Cij, T cthr, long N, long H, long Mc, long h) {
+                            const T *Cij, T cthr, long N, long H, long Mc, long h, int *rows, int *row_cnt,
+                            long cap) {
   SB_REQUIRE(W && wmask && Ci && Cj && Cij, "null pointer");
   SB_REQUIRE(h >= 0 && h < H, "hypercolumn index out of range");
+  SB_REQUIRE(!rows || (row_cnt && cap > 0 && cap % 16 == 0), "row list arguments");
+  SB_REQUIRE(cdiv(N * Mc, 256) + 1 < (1L << 31), "too many elements for one launch");
   const TraceScalars<T> s = TraceScalars<T>::from(T(0), cthr);
   ProfScope prof_(st, K_MASK_FIX);
-  hipLaunchKernelGGL((k_mask_fix_weights<T>), dim3((unsigned)cdiv(N * Mc, 256)), dim3(256), 0, st, W,
-                     wmask, Ci, Cj, Cij, cthr, s.cthr4, N, H * Mc, H, Mc, h);
+  // with a row list, one more workgroup rebuilds the list of hypercolumn h
+  hipLaunchKernelGGL((k_mask_fix_weights<T>), dim3((unsigned)(cdiv(N * Mc, 256) + (rows ? 1 : 0))), dim3(256), 0,
+                     st, W, wmask, Ci, Cj, Cij, cthr, s.cthr4, N, H * Mc, H, Mc, h, rows, row_cnt, cap);
   SB_LAUNCH_CHECK();
   return 0;
 }
@@ -340,7 +344,7 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
   template int launch_update_mask<T>(hipStream_t, uint8_t *, const T *, const T *, const T *,         \
                                      const T *, T, long, long, long, long, long, T *, int *);         \
   template int launch_mask_fix_weights<T>(hipStream_t, T *, const uint8_t *, const T *, const T *,    \
-                                          const T *, T, long, long, long, long);                      \
+                                          const T *, T, long, long, long, long, int *, int *, long);  \
   template int launch_apply_mask<T>(hipStream_t, T *, const uint8_t *, long, long, long);             \
   template int launch_argmax_rows<T>(hipStream_t, const T *, const T *, long, long, int32_t *,        \
                                      unsigned long long *);                                           \

@@ -268,10 +268,9 @@ static int layer_train_step(Layer &L, const T *x, const T *y, long B, long h) {
                                (const T *)L.Cij, cthr, L.N, L.H, L.Mc, h, 16, (T *)L.nom, L.csum);
     if (rc) return rc;
     rc = launch_mask_fix_weights<T>(st, (T *)L.W, L.wmask, (const T *)L.Ci, (const T *)L.Cj,
-                                    (const T *)L.Cij, cthr, L.N, L.H, L.Mc, h);
-    if (rc) return rc;
-    // a swap leaves the number of connected rows of the hypercolumn as it was, so the list fits
-    if (L.rows) rc = launch_mask_rows(st, L.rows, L.row_cnt, L.wmask, L.N, L.H, L.rows_cap, h, 1);
+                                    (const T *)L.Cij, cthr, L.N, L.H, L.Mc, h, L.rows, L.row_cnt,
+                                    L.rows_cap);
+    // (a swap leaves the number of connected rows of the hypercolumn as it was, so its list still fits)
     if (rc) return rc;
   }
   return 0;
@@ -642,7 +641,8 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
     rc = launch_update_mask<T>(g_ctx.stream, wmask, (const T *)nullptr, Ci, Cj, Cij, cthr, N, H, Mc,   \
                                h, 16, (T *)g_ctx.mask_nom, g_ctx.mask_csum);                           \
     if (rc) return rc;                                                                                 \
-    return launch_mask_fix_weights<T>(g_ctx.stream, W, wmask, Ci, Cj, Cij, cthr, N, H, Mc, h);         \
+    return launch_mask_fix_weights<T>(g_ctx.stream, W, wmask, Ci, Cj, Cij, cthr, N, H, Mc, h, nullptr, \
+                                      nullptr, 0);                                                     \
   }
 
 SB_DEFINE_KERNEL_API(f32, float)
