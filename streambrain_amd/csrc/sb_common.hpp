@@ -97,64 +97,6 @@ __device__ __forceinline__ void load_vw(T (&out)[Real<T>::VW], const T *row, lon
   }
 }
 
-template <typename T, bool VEC>
-__device__ __forceinline__ void store_vw(const T (&in)[Real<T>::VW], T *row, long col, long limit) {
-  constexpr int VW = Real<T>::VW;
-  if (VEC) {
-    if (col < limit) {
-      typename Real<T>::vec_t v;
-#pragma unroll
-      for (int e = 0; e < VW; e++) v[e] = in[e];
-      *reinterpret_cast<typename Real<T>::vec_t *>(row + col) = v;
-    }
-  } else {
-#pragma unroll
-    for (int e = 0; e < VW; e++)
-      if (col + e < limit) row[col + e] = in[e];
-  }
-}
-
-// Branch-free load for software-pipelined loops: the 16-byte load is always issued (from `p` when ok,
-// from the always-valid, 16-byte aligned `safe` otherwise) and the result zeroed afterwards, so the
-// compiler keeps several of them in flight with exact wait counts instead of fencing a guarded load.
-template <typename T>
-__device__ __forceinline__ void load_vw_sel(T (&out)[Real<T>::VW], const T *p, const T *safe, bool ok) {
-  constexpr int VW = Real<T>::VW;
-  const typename Real<T>::vec_t v = *reinterpret_cast<const typename Real<T>::vec_t *>(ok ? p : safe);
-#pragma unroll
-  for (int e = 0; e < VW; e++) out[e] = ok ? v[e] : T(0);
-}
-
-// Branch-free loads in two halves, for code that wants many loads in flight before the first use.
-// load_vw_raw issues the loads of base[off + col .. off + col + VW) -- from element 0 of the array where
-// the guard fails, so `base` must point to at least one valid (for VEC: 16-byte aligned) vector -- and
-// zero_invalid, called where the values are consumed, zeroes what the guard excludes.  (A select right
-// behind the load would make the compiler wait for the load there.)
-template <typename T, bool VEC>
-__device__ __forceinline__ void load_vw_raw(T (&out)[Real<T>::VW], const T *base, long off, long col,
-                                            long limit, bool row_ok) {
-  constexpr int VW = Real<T>::VW;
-  if (VEC) {
-    const bool ok = row_ok && col < limit;
-    const typename Real<T>::vec_t v =
-        *reinterpret_cast<const typename Real<T>::vec_t *>(base + (ok ? off + col : 0));
-#pragma unroll
-    for (int e = 0; e < VW; e++) out[e] = v[e];
-  } else {
-#pragma unroll
-    for (int e = 0; e < VW; e++) out[e] = base[(row_ok && col + e < limit) ? off + col + e : 0];
-  }
-}
-template <typename T, bool VEC>
-__device__ __forceinline__ void zero_invalid(T (&v)[Real<T>::VW], long col, long limit, bool row_ok) {
-  constexpr int VW = Real<T>::VW;
-#pragma unroll
-  for (int e = 0; e < VW; e++) {
-    const bool ok = VEC ? (row_ok && col < limit) : (row_ok && col + e < limit);
-    v[e] = ok ? v[e] : T(0);
-  }
-}
-
 // A bounds-checked window of at most 2 GiB onto a global array, addressed through a buffer descriptor
 // with 32-bit byte offsets: a per-lane offset plus a wavefront-uniform one that lives in a scalar
 // register.  Accesses past the end of the window read zero and store nothing, in hardware; so a loop
@@ -199,22 +141,22 @@ struct BufferWindow {
     }
   }
   // NE consecutive elements (4, 8, 12 or 16 bytes) as one access; element-aligned
-  template <int NE, int AUX = 0>
+  template <int NE>
   __device__ __forceinline__ void load_n(T (&out)[NE], unsigned at) const {
     constexpr int BYTES = NE * (int)sizeof(T);
     static_assert(BYTES == 4 || BYTES == 8 || BYTES == 12 || BYTES == 16, "one buffer access");
     using u3 = unsigned __attribute__((ext_vector_type(3)));
     unsigned raw[BYTES / 4];
     if constexpr (BYTES == 4) {
-      raw[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)at, 0, AUX);
+      raw[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)at, 0, 0);
     } else if constexpr (BYTES == 8) {
-      const u2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)at, 0, AUX);
+      const u2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)at, 0, 0);
       raw[0] = v[0], raw[1] = v[1];
     } else if constexpr (BYTES == 12) {
-      const u3 v = __builtin_amdgcn_raw_buffer_load_b96(rsrc, (int)at, 0, AUX);
+      const u3 v = __builtin_amdgcn_raw_buffer_load_b96(rsrc, (int)at, 0, 0);
       raw[0] = v[0], raw[1] = v[1], raw[2] = v[2];
     } else {
-      const u4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)at, 0, AUX);
+      const u4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)at, 0, 0);
       raw[0] = v[0], raw[1] = v[1], raw[2] = v[2], raw[3] = v[3];
     }
     __builtin_memcpy(out, raw, BYTES);
@@ -241,41 +183,6 @@ struct BufferWindow {
     }
   }
 };
-
-// Width-generic variants: W consecutive elements (W = 1, 2, 4 for float; 1, 2 for double), moved as one
-// W*sizeof(T)-byte access when VEC promises that alignment and limit % W == 0.
-template <typename T, int W>
-struct VecOf {
-  typedef T type __attribute__((ext_vector_type(W)));
-};
-template <typename T, int W, bool VEC>
-__device__ __forceinline__ void load_w(T (&out)[W], const T *row, long col, long limit, bool row_ok) {
-  if (VEC && W > 1) {
-    typename VecOf<T, (W > 1 ? W : 2)>::type v = {};
-    if (row_ok && col < limit)
-      v = *reinterpret_cast<const typename VecOf<T, (W > 1 ? W : 2)>::type *>(row + col);
-#pragma unroll
-    for (int e = 0; e < W; e++) out[e] = v[e];
-  } else {
-#pragma unroll
-    for (int e = 0; e < W; e++) out[e] = (row_ok && col + e < limit) ? row[col + e] : T(0);
-  }
-}
-template <typename T, int W, bool VEC>
-__device__ __forceinline__ void store_w(const T (&in)[W], T *row, long col, long limit) {
-  if (VEC && W > 1) {
-    if (col < limit) {
-      typename VecOf<T, (W > 1 ? W : 2)>::type v;
-#pragma unroll
-      for (int e = 0; e < W; e++) v[e] = in[e];
-      *reinterpret_cast<typename VecOf<T, (W > 1 ? W : 2)>::type *>(row + col) = v;
-    }
-  } else {
-#pragma unroll
-    for (int e = 0; e < W; e++)
-      if (col + e < limit) row[col + e] = in[e];
-  }
-}
 
 // The weight of one synapse from its traces, shared by the trace/weight kernel and the rewiring
 // kernels so both see bit-identical values:  log(max(cij, cthr^4) / (ci * cj)) evaluated as

@@ -16,18 +16,21 @@
 //      each wavefront feeds its 32 x 32 sub-tile (2 x 2 MFMA blocks) with two 8-byte LDS reads per K
 //      step of 4.  The global loads of chunk c+1 are issued before chunk c is consumed.
 //   2. From the same LDS slabs, the lanes of one wavefront add up one column each of x, those of
-//      another one column each of y, in batch order b = 0..B-1 without FMA contraction: the reference's summation order, so Ci, Cj and
-//      kbi stay bit-exact against a strict-IEEE build of it.  Every tile needs Ci for its rows and Cj
+//      another one column each of y (which two wavefronts rotates with the tile index), in batch order
+//      b = 0..B-1 without FMA contraction: the reference's summation order, so Ci, Cj and kbi stay
+//      bit-exact against a strict-IEEE build of it.  Every tile needs Ci for its rows and Cj
 //      for its columns, so every workgroup recomputes them from the OLD traces (a tile row shares x,
 //      a tile column shares y: same inputs, same order, same bits).  The old traces are read from
 //      Ci/Cj and the new ones written to Ci_next/Cj_next by the tiles of the first tile column / row:
 //      no workgroup ever reads a value another one is writing.
 //   3. Global loads return in issue order, so the Cij tile (HBM latency) is requested only while the
 //      second-to-last chunk is being multiplied: the MFMA loop never waits for it, and it has arrived
-//      by the time the epilogue needs it.  All loads are branch-free (clamped addresses): a guarded
-//      load makes the compiler wait for every outstanding load at the join.
+//      by the time the epilogue needs it.  All loads are branch-free (bounds-checked buffer windows
+//      instead of guards): a guarded load makes the compiler wait for every outstanding load at the
+//      join.
 //   4. The accumulators go through LDS into a row-major layout; each thread then finishes VW consecutive
-//      columns of 4 rows: decay + clamp, weight, mask, one 16-byte store each to Cij and W.
+//      columns of 4 rows: decay + clamp, weight, mask, one 16-byte store each to Cij and W.  With
+//      w_masked, a wavefront whose vectors of a pass all lie under zero mask bytes skips the weight.
 #pragma once
 #include <type_traits>
 
@@ -98,9 +101,6 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   const int eg = tid % G, er = tid / G;
   const long ecol = j0 + VW * eg;
 
-#ifdef SB_STAGGER
-  for (int z = 0; z < (int)(blockIdx.x / 256) * SB_STAGGER; z++) __builtin_amdgcn_s_sleep(16);
-#endif
   SB_PHASE_MARK(0);
   // x, y, the Cij tile and the W tile are reached through bounds-checked buffer windows: rows past the
   // batch or past the matrix read zero / store nothing in hardware, so there are no clamped addresses,
