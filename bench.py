@@ -2,6 +2,7 @@
 """Benchmark of the BCPNN layer training step on one MI355X.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+  python bench.py --workload stl10|largest|wide64     (other configurations, see LARGE below)
 
 Workload: the MNIST-shaped 2-layer network, float32, batch 128, 60000 seeded
 synthetic samples; input 784 pixels complementary-coded to 1568 units (~19% nonzero pixels, uniform
@@ -190,6 +191,104 @@ def cpu_baseline(x, y, budget_s=15.0, max_steps=100000):
             "ms_per_step": 1e3 * dt / max(steps, 1)}
 
 
+# Other layer shapes, run through the same network path (one structural-plasticity layer, data resident in
+# HBM, first epoch: no rewiring).  in_features, hypercolumns, minicolumns, batch, mask density, dtype,
+# samples kept on the device (an epoch of the run cycles through them), fraction of non-zero inputs.
+LARGE = {
+    "stl10": dict(n=55296, h=200, mc=100, batch=256, density=0.05, dtype=np.float32, samples=5000, nonzero=1.0,
+                  what="configs[3]: STL-10-shaped layer 55296 -> 200x100, float32, batch 256, mask density 0.05"),
+    "largest": dict(n=65536, h=1000, mc=100, batch=1024, density=1.0, dtype=np.float32, samples=4096, nonzero=0.2,
+                    what="configs[4]: 65536 -> 1000x100, float32, batch 1024, binary inputs, dense mask"),
+    "wide64": dict(n=1568, h=100, mc=100, batch=512, density=0.1, dtype=np.float64, samples=60000, nonzero=0.19,
+                   what="configs[2]: 1568 -> 100x100, float64, batch 512, mask density 0.1"),
+}
+
+
+def large_workload(name, steps, warmup):
+    """Training steps of one structural-plasticity layer of a LARGE shape; prints one JSON line of the same
+    form as the headline run (no CPU baseline: the oracle needs minutes per step at these sizes)."""
+    from streambrain_amd import _capi
+    cfg = LARGE[name]
+    n, h, mc, batch, dt = cfg["n"], cfg["h"], cfg["mc"], cfg["batch"], cfg["dtype"]
+    m, ns, es = h * mc, cfg["samples"], np.dtype(cfg["dtype"]).itemsize
+    rng = np.random.default_rng(1000 + len(name))
+    if name == "largest":
+        x = (rng.random((ns, n), dtype=np.float32) < cfg["nonzero"]).astype(dt)
+    else:
+        half = n // 2
+        px = rng.random((ns, half), dtype=np.float32)
+        if cfg["nonzero"] < 1.0:
+            px *= rng.random((ns, half), dtype=np.float32) < cfg["nonzero"]
+        x = np.concatenate([px, 1.0 - px], axis=1).astype(dt)
+    lib = _capi.lib()
+    _capi.init(0)
+    c = _capi.check
+    net = ctypes.c_void_p()
+    c(lib.sb_net_create(ctypes.byref(net), 0 if dt == np.float32 else 1))
+    tau = HP["l1_taupdt"] * np.sqrt(batch / 128.0)
+    c(lib.sb_net_add_plastic_layer(net, n, h, mc, tau, HP["l1_pmin"], HP["l1_khalf"], HP["l1_taubdt"], 1.0,
+                                   1.0 / mc, 1.0 / mc))
+    # a (never trained) output layer behind it, so that the layer trains on its own activation
+    c(lib.sb_net_add_dense_layer(net, m, 1, N_OUT, HP["l2_taupdt"], 1.0 / mc, 1.0 / N_OUT, 1.0 / mc / N_OUT))
+    connected = n * h
+    if cfg["density"] < 1.0:
+        wmask = (rng.random((n, h), dtype=np.float32) < cfg["density"]).astype(np.uint8)
+        connected = int(np.count_nonzero(wmask))
+        c(lib.sb_net_set_layer_state(net, 0, b"wmask", wmask.ctypes.data, wmask.nbytes))
+    c(lib.sb_net_set_training_data(net, x.ctypes.data, None, ns, n, 0))
+    nb = (ns + batch - 1) // batch
+
+    def run(first, count):
+        done = 0
+        for epoch, fb, take in batch_plan(first, count, nb):
+            perm = rng.permutation(ns).astype(np.int64) if fb == 0 else None
+            hc = rng.permutation(h).astype(np.int64)
+            c(lib.sb_net_train_batches(net, 0, batch, perm.ctypes.data if perm is not None else None,
+                                       hc.ctypes.data, 0, fb, take, 0))
+            done += sum(min(batch, ns - b * batch) for b in range(fb, fb + take))
+        return done
+
+    warmup = max(warmup, 1)
+    warmup += (-warmup) % nb  # the timed region starts at an epoch boundary
+    run(0, warmup)
+    c(lib.sb_sync())
+    t0 = time.perf_counter()
+    samples = run(warmup, steps)
+    c(lib.sb_sync())
+    dt_s = time.perf_counter() - t0
+    c(lib.sb_profile_start())
+    run(warmup + steps + (-(warmup + steps)) % nb, min(steps, nb))
+    c(lib.sb_profile_stop())
+    kernels = {}
+    for k in range(lib.sb_profile_kernels()):
+        ms, cnt = ctypes.c_double(0), ctypes.c_long(0)
+        c(lib.sb_profile_get(k, ctypes.byref(ms), ctypes.byref(cnt)))
+        if cnt.value:
+            kernels[lib.sb_profile_kernel_name(k).decode()] = {"launches": cnt.value,
+                                                               "avg_us": 1e3 * ms.value / cnt.value}
+    tw = kernels.get("train_fused", {"avg_us": float("nan")})["avg_us"] * 1e-6
+    fw = kernels.get("forward", {"avg_us": float("nan")})["avg_us"] * 1e-6
+    peak = 157.3 if dt == np.float32 else 78.6
+    gemm = 2.0 * batch * n * m  # the Cij trace GEMM of a full batch; bound: MFMA at these batch sizes
+    fwd_flops = 2.0 * batch * connected * mc if cfg["density"] <= 0.5 else gemm
+    print(json.dumps({
+        "metric": "train samples/sec on 1 MI355X; % HBM / MFMA peak",
+        "value": samples / dt_s, "unit": "samples/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": 1e3 * dt_s / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if dt == np.float32 else "f64", "data": "synthetic",
+        "config": {"workload": cfg["what"], "batch": batch, "in_features": n, "hypercolumns": h,
+                   "minicolumns": mc, "samples": ns},
+        "roofline": {"bound": "mfma", "kernel": "k_train_fused", "achieved": gemm / tw / 1e12, "peak": peak,
+                     "unit": "TFLOP/s", "frac": gemm / tw / 1e12 / peak, "traffic": None,
+                     "algorithmic_flops_per_launch": gemm, "avg_launch_us": tw * 1e6,
+                     "bytes_3sNM_per_launch": 3 * es * n * m, "achieved_GBps_on_3sNM": 3 * es * n * m / tw / 1e9},
+        "mfma": {"kernel": "k_forward_rows" if cfg["density"] <= 0.5 else "k_forward",
+                 "flops_per_launch": fwd_flops, "achieved_tflops": fwd_flops / fw / 1e12, "peak_tflops": peak,
+                 "frac": fwd_flops / fw / 1e12 / peak, "avg_launch_us": fw * 1e6},
+        "kernels": kernels, "cpu_baseline": None}))
+    return 0
+
+
 def measured_traffic():
     """HBM bytes per launch of the dominant kernel, as measured with rocprofv3 --pmc FETCH_SIZE /
     WRITE_SIZE and recorded in profiles/ (line `traffic_bytes_per_launch: N`); None when absent."""
@@ -226,6 +325,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=60)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--samples", type=int, default=N_SAMPLES)
+    ap.add_argument("--workload", choices=["mnist"] + sorted(LARGE), default="mnist",
+                    help="mnist (default): the headline configuration; the others: one layer of a larger "
+                         "shape (--steps defaults to two epochs of its resident samples)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run six 64 MiB device-to-device copies: the known-size kernel that "
                          "hardware counter readings (FETCH_SIZE, WRITE_SIZE) are scaled by")
@@ -237,6 +339,11 @@ def main():
 
     if args.copy_calibration:
         return copy_calibration()
+    if args.workload != "mnist":
+        cfg = LARGE[args.workload]
+        nb = (cfg["samples"] + cfg["batch"] - 1) // cfg["batch"]
+        steps = args.steps if "--steps" in sys.argv else 2 * nb
+        return large_workload(args.workload, steps, args.warmup if "--warmup" in sys.argv else nb)
 
     x, y = synthetic_dataset(args.samples)
     run = GpuRun(x, y)
