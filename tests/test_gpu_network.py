@@ -262,3 +262,38 @@ def test_checkpoint_round_trip_on_device(hb, tmp_path):
     other.fit(X, Y, 32, [(0, 1)])
     assert np.array_equal(net._layers[0].weights, other._layers[0].weights)
     assert np.array_equal(net._layers[0].wmask, other._layers[0].wmask)
+
+
+@pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-5), (np.float64, 1e-12)])
+def test_forward_over_connected_rows_tracks_the_state(hb, dtype, tol):
+    """A sparse layer's forward pass runs over its lists of connected rows once a training step has
+    left W masked, and over all rows again after W or the mask has been written from outside: all of
+    these must agree with the dense computation on the state read back from the device."""
+    from streambrain_amd import kernels_hip as k
+    rng = np.random.default_rng(5)
+    X = synthetic_images(rng, 3 * 64, 200)
+    Y = one_hot_labels(rng, X.shape[0], 10)
+    net = build_two_layer(hb, 400, 6, 20, 10, MNIST_HP, dtype, seed=3, density=0.2)
+    layer = net._layers[0]
+    xt = np.ascontiguousarray(X[:40].astype(dtype))
+
+    def dense(W, b):
+        return k.compute_activation(np.ascontiguousarray(W), np.ascontiguousarray(b), xt, 6, 20)
+
+    # before any training step W is the unmasked initial draw: dense path
+    assert rel_err(net.forward(xt, last_layer=0), dense(layer.weights, layer.bias)) <= 4 * tol
+    net.fit(X, Y, 64, [(0, 2)])  # two epochs, the second with rewiring
+    W, b, mask = layer.weights, layer.bias, layer.wmask
+    assert np.all(W[np.repeat(mask, 20, axis=1) == 0] == 0)
+    assert rel_err(net.forward(xt, last_layer=0), dense(W, b)) <= 4 * tol  # row lists (after rewiring)
+    # an unmasked W written from outside must be used as it is
+    W2 = (W + 0.01).astype(dtype)
+    layer.weights = W2
+    assert rel_err(net.forward(xt, last_layer=0), dense(W2, b)) <= 4 * tol
+    # ... and a new mask does not touch W until the next training step
+    layer.wmask = np.ascontiguousarray(1 - mask)
+    assert rel_err(net.forward(xt, last_layer=0), dense(W2, b)) <= 4 * tol
+    net.fit(X, Y, 64, [(0, 1)])
+    W3, mask3 = layer.weights, layer.wmask
+    assert np.all(W3[np.repeat(mask3, 20, axis=1) == 0] == 0)
+    assert rel_err(net.forward(xt, last_layer=0), dense(W3, layer.bias)) <= 4 * tol
