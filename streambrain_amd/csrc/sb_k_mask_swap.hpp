@@ -149,14 +149,31 @@ __device__ __forceinline__ KeyIdx<K> dpp_keyidx(KeyIdx<K> c) {
   return KeyIdx<K>{dpp_move_k<CTRL>(c.key), dpp_move<CTRL>(c.idx)};
 }
 template <typename K>
-__device__ __forceinline__ KeyIdx<K> wave_pick(KeyIdx<K> c) {  // every lane ends with the result
+__device__ __forceinline__ KeyIdx<K> wave_pick(KeyIdx<K> c) {  // the result is wavefront-uniform
   c = pick_key<K>(c, dpp_keyidx<K, kDppSwap1>(c));
   c = pick_key<K>(c, dpp_keyidx<K, kDppSwap2>(c));
   c = pick_key<K>(c, dpp_keyidx<K, kDppHalfMirror>(c));
   c = pick_key<K>(c, dpp_keyidx<K, kDppMirror>(c));
-#pragma unroll
-  for (int o = 16; o <= 32; o <<= 1) c = pick_key<K>(c, KeyIdx<K>{(K)__shfl_xor(c.key, o), __shfl_xor(c.idx, o)});
-  return c;
+  // every lane of a row of 16 now holds its row's pick; the four rows are combined from scalar
+  // registers (a lane read is far cheaper than an exchange through the LDS crossbar)
+  const KeyIdx<K> r0{readlane_k(c.key, 0), __builtin_amdgcn_readlane(c.idx, 0)};
+  const KeyIdx<K> r1{readlane_k(c.key, 16), __builtin_amdgcn_readlane(c.idx, 16)};
+  const KeyIdx<K> r2{readlane_k(c.key, 32), __builtin_amdgcn_readlane(c.idx, 32)};
+  const KeyIdx<K> r3{readlane_k(c.key, 48), __builtin_amdgcn_readlane(c.idx, 48)};
+  return pick_key<K>(pick_key<K>(r0, r1), pick_key<K>(r2, r3));
+}
+
+// 32-bit keys: (key, index + 1) packed into one 64-bit integer whose unsigned order is the order pick_key
+// defines (0 = no candidate), so a pick is a 64-bit maximum: a third of the instructions.
+__device__ __forceinline__ KeyIdx<uint32_t> wave_pick(KeyIdx<uint32_t> c) {
+  uint64_t v = c.idx < 0 ? 0ull : ((uint64_t)c.key << 32) | (uint32_t)(c.idx + 1);
+  auto larger = [](uint64_t a, uint64_t b) { return b > a ? b : a; };
+  v = larger(v, dpp_move_k<kDppSwap1>(v));
+  v = larger(v, dpp_move_k<kDppSwap2>(v));
+  v = larger(v, dpp_move_k<kDppHalfMirror>(v));
+  v = larger(v, dpp_move_k<kDppMirror>(v));
+  const uint64_t m = larger(larger(readlane_k(v, 0), readlane_k(v, 16)), larger(readlane_k(v, 32), readlane_k(v, 48)));
+  return KeyIdx<uint32_t>{(uint32_t)(m >> 32), (int)(uint32_t)m - 1};
 }
 
 template <typename T, int NT, int R>
@@ -168,7 +185,8 @@ struct MaskSwapFast {
   static_assert(NT * R <= (BINS << 2) && BINS % NT == 0, "row indices must fit the index histogram");
   struct Shared {
     unsigned hist[2][BINS];
-    int cand[2][64];
+    int cand[2][64], cand_cs[2][64];  // candidate rows, their connection counts ...
+    T cand_nom[2][64];                // ... and score nominators
     int ncand[2], sel_bin[2], sel_above[2], wtot[2][NWV];
     K eq_min[2], eq_max[2];
   };
@@ -219,7 +237,8 @@ struct MaskSwapFast {
   }
 
   // true: the swaps are done and written back; false: nothing was changed, run the full scan
-  static __device__ bool run(const MaskArgs<T> &a, Shared &sh, const T (&score)[R], const int (&m)[R]) {
+  static __device__ bool run(const MaskArgs<T> &a, Shared &sh, const T (&score)[R], const int (&m)[R],
+                             const T (&nom)[R], const int (&cs)[R]) {
     const int tid = threadIdx.x, lane = tid & 63;
     K key[R];
 #pragma unroll
@@ -272,7 +291,7 @@ struct MaskSwapFast {
       const K top = key[k] >> TAIL;
       if (all[g] || top >= prefix[g]) {
         const int pos = atomicAdd(&sh.ncand[g], 1);
-        if (pos < 64) sh.cand[g][pos] = tid + NT * k;
+        if (pos < 64) sh.cand[g][pos] = tid + NT * k, sh.cand_cs[g][pos] = cs[k], sh.cand_nom[g][pos] = nom[k];
       }
       if (!all[g] && top == prefix[g]) {
         atomicMin(&sh.eq_min[g], key[k]);
@@ -310,7 +329,7 @@ struct MaskSwapFast {
         const int i = tid + NT * k;
         if (top > prefix[g] || (top == prefix[g] && (i >> ISH) >= sh.sel_bin[g])) {
           const int pos = atomicAdd(&sh.ncand[g], 1);
-          if (pos < 64) sh.cand[g][pos] = i;
+          if (pos < 64) sh.cand[g][pos] = i, sh.cand_cs[g][pos] = cs[k], sh.cand_nom[g][pos] = nom[k];
         }
       }
       __syncthreads();
@@ -325,15 +344,15 @@ struct MaskSwapFast {
     int nS = sh.ncand[0], nA = sh.ncand[1];
     bool vS = lane < nS, vA = lane < nA;
     int iS = vS ? sh.cand[0][lane] : 0, iA = vA ? sh.cand[1][lane] : 0;
-    int csS = a.csum[iS], csA = a.csum[iA];
-    const T nomS = a.nom[iS], nomA = a.nom[iA];
+    int csS = vS ? sh.cand_cs[0][lane] : 0, csA = vA ? sh.cand_cs[1][lane] : 0;
+    const T nomS = vS ? sh.cand_nom[0][lane] : T(0), nomA = vA ? sh.cand_nom[1][lane] : T(0);
     // keys as seen from the silent side (largest score wins) and from the active side (smallest wins)
     K kS = SK::of(mask_score<T>(nomS, csS)), kS_other = (K)~SK::of(mask_score<T>(nomS, csS + 1));
     K kA = (K)~SK::of(mask_score<T>(nomA, csA)), kA_other = SK::of(mask_score<T>(nomA, csA - 1));
     for (long it = 0; it < a.iterations; it++) {
       KeyIdx<K> cmax{kS, vS ? iS : -1}, cmin{kA, vA ? iA : -1};
-      cmax = wave_pick<K>(cmax);
-      cmin = wave_pick<K>(cmin);
+      cmax = wave_pick(cmax);
+      cmin = wave_pick(cmin);
       if (cmax.idx < 0 || cmin.idx < 0) break;  // no silent or no active row
       if (cmax.key < (K)~cmin.key) break;       // vmax0 < vmin1
       const int lS = __builtin_ctzll(__ballot(vS && iS == cmax.idx));
@@ -399,7 +418,7 @@ __global__ __launch_bounds__(NT) void k_mask_swap_reg(MaskArgs<T> a) {
   const bool track_first = __syncthreads_or(has_nan) != 0;
   if (!track_first && a.iterations <= MaskSwapFast<T, NT, R>::TOPK) {
     __shared__ typename MaskSwapFast<T, NT, R>::Shared fast_lds;
-    if (MaskSwapFast<T, NT, R>::run(a, fast_lds, score, m)) return;
+    if (MaskSwapFast<T, NT, R>::run(a, fast_lds, score, m, nom, cs)) return;
     __syncthreads();
   }
 
