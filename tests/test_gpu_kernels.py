@@ -71,6 +71,7 @@ def test_mask_rows(k, N, H, density):
                                               (7, 40, 3, 12, 0.3), (33, 300, 2, 200, 0.2),
                                               (16, 64, 2, 64, 1.0), (20, 100, 2, 256, 0.05),
                                               (5, 50, 3, 12, 0.0), (300, 5000, 4, 100, 0.4),
+                                              (20, 6000, 2, 64, 0.5),  # lists longer than one LDS segment
                                               (12, 40, 2, 224, 0.5)])
 def test_compute_activation_rows(k, oracle, dtype, B, N, H, Mc, density):
     """The row-list forward kernel against the dense reference computation on the masked weights."""
