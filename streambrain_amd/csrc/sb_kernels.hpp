@@ -79,6 +79,22 @@ __global__ __launch_bounds__(256) void k_apply_mask(T *W, const uint8_t *wmask, 
   }
 }
 
+// Counts the entries of W that are not +0 / -0 although their mask byte is 0 (0 means: W is in the state
+// apply_mask leaves behind).  NaN counts as non-zero.
+template <typename T>
+__global__ __launch_bounds__(256) void k_count_unmasked(const T *W, const uint8_t *wmask, long N, long M,
+                                                        long H, long Mc, unsigned long long *count) {
+  const long total = N * M;
+  const long stride = (long)gridDim.x * 256;
+  unsigned long long mine = 0;
+  for (long e = (long)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+    const long i = e / M;
+    const long j = e - i * M;
+    mine += (wmask[i * H + j / Mc] == 0 && !(W[e] == T(0))) ? 1 : 0;
+  }
+  if (__syncthreads_or(mine != 0) && mine != 0) atomicAdd(count, mine);
+}
+
 // =====================================================================================================
 // Structural-plasticity rewiring of one hypercolumn                      omp.cc:248-320
 // Step 1 (k_mask_scores): per input row, the score nominator over the Mc columns of hypercolumn h and

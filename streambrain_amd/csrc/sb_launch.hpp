@@ -100,6 +100,9 @@ int launch_mask_fix_weights(hipStream_t st, T *W, const uint8_t *wmask, const T 
 template <typename T>
 int launch_apply_mask(hipStream_t st, T *W, const uint8_t *wmask, long N, long H, long Mc);
 template <typename T>
+int launch_count_unmasked(hipStream_t st, const T *W, const uint8_t *wmask, long N, long H, long Mc,
+                          unsigned long long *count);
+template <typename T>
 int launch_argmax_rows(hipStream_t st, const T *act, const T *labels, long B, long M, int32_t *pred,
                        unsigned long long *correct);
 template <typename T>

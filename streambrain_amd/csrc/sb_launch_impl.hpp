@@ -292,6 +292,21 @@ int launch_apply_mask(hipStream_t st, T *W, const uint8_t *wmask, long N, long H
   return 0;
 }
 
+// *count += number of entries of W that are non-zero under a zero mask byte
+template <typename T>
+int launch_count_unmasked(hipStream_t st, const T *W, const uint8_t *wmask, long N, long H, long Mc,
+                          unsigned long long *count) {
+  SB_REQUIRE(W && wmask && count, "null pointer");
+  SB_REQUIRE(N > 0 && H > 0 && Mc > 0, "sizes must be positive");
+  const long total = N * H * Mc;
+  const long blocks = cdiv(total, 1024) < 8192 ? cdiv(total, 1024) : 8192;
+  ProfScope prof_(st, K_APPLY_MASK);
+  hipLaunchKernelGGL((k_count_unmasked<T>), dim3((unsigned)blocks), dim3(256), 0, st, W, wmask, N, H * Mc, H,
+                     Mc, count);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
 // ------------------------------------------------------------------------------------- classification
 template <typename T>
 int launch_argmax_rows(hipStream_t st, const T *act, const T *labels, long B, long M, int32_t *pred,
@@ -346,6 +361,8 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
   template int launch_mask_fix_weights<T>(hipStream_t, T *, const uint8_t *, const T *, const T *,    \
                                           const T *, T, long, long, long, long, int *, int *, long);  \
   template int launch_apply_mask<T>(hipStream_t, T *, const uint8_t *, long, long, long);             \
+  template int launch_count_unmasked<T>(hipStream_t, const T *, const uint8_t *, long, long, long,    \
+                                        unsigned long long *);                                        \
   template int launch_argmax_rows<T>(hipStream_t, const T *, const T *, long, long, int32_t *,        \
                                      unsigned long long *);                                           \
   template int launch_gather_rows<T>(hipStream_t, T *, const T *, const int64_t *, long, long);       \

@@ -160,6 +160,7 @@ struct Layer {
   int *rows = nullptr, *row_cnt = nullptr;
   long rows_cap = 0;
   bool w_masked = false;
+  bool w_unchecked = false;  // W or wmask came from outside and has not been looked at yet
 };
 
 }  // namespace sb
@@ -174,7 +175,8 @@ struct sb_net {
   int64_t *d_perm = nullptr;
   int64_t *h_perm = nullptr;  // pinned staging
   hipEvent_t perm_copied = nullptr;
-  unsigned long long *d_correct = nullptr;
+  unsigned long long *d_correct = nullptr;   // evaluate's counter
+  unsigned long long *d_unmasked = nullptr;  // layer_check_masked's counter
 };
 
 namespace sb {
@@ -237,8 +239,29 @@ static int ensure_act(sb_net *net, long rows) {
   return 0;
 }
 
+// After W or wmask of a layer with row lists has been written from outside (a restored checkpoint, say),
+// one pass over W tells whether it is zero under every zero mask byte, i.e. whether the forward pass may
+// walk the row lists right away.  Costs one read of W and a host round trip, once per such write.
 template <typename T>
-static int layer_forward(const Layer &L, const T *x, long B) {
+static int layer_check_masked(sb_net *net, Layer &L) {
+  L.w_unchecked = false;
+  if (!L.rows || L.w_masked) return 0;
+  unsigned long long count = 0;
+  SB_HIP(hipMemcpyAsync(net->d_unmasked, &count, sizeof(count), hipMemcpyHostToDevice, g_ctx.stream));
+  int rc = launch_count_unmasked<T>(g_ctx.stream, (const T *)L.W, L.wmask, L.N, L.H, L.Mc, net->d_unmasked);
+  if (rc) return rc;
+  SB_HIP(hipMemcpyAsync(&count, net->d_unmasked, sizeof(count), hipMemcpyDeviceToHost, g_ctx.stream));
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  L.w_masked = count == 0;
+  return 0;
+}
+
+template <typename T>
+static int layer_forward(sb_net *net, Layer &L, const T *x, long B) {
+  if (L.w_unchecked) {
+    int rc = layer_check_masked<T>(net, L);
+    if (rc) return rc;
+  }
   if (L.rows && L.w_masked)
     return launch_forward_rows<T>(g_ctx.stream, (T *)L.act, x, (const T *)L.W, (const T *)L.bias, L.rows,
                                   L.row_cnt, L.rows_cap, B, L.N, L.H, L.Mc);
@@ -262,7 +285,7 @@ static int layer_train_step(Layer &L, const T *x, const T *y, long B, long h) {
   if (rc) return rc;
   std::swap(L.Ci, L.Ci_alt);
   std::swap(L.Cj, L.Cj_alt);
-  if (L.plastic) L.w_masked = true;  // every entry of W has just been written under the mask
+  if (L.plastic) L.w_masked = true, L.w_unchecked = false;  // every entry of W has just been written under the mask
   if (L.plastic && h >= 0) {
     rc = launch_update_mask<T>(st, L.wmask, (const T *)nullptr, (const T *)L.Ci, (const T *)L.Cj,
                                (const T *)L.Cij, cthr, L.N, L.H, L.Mc, h, 16, (T *)L.nom, L.csum);
@@ -282,6 +305,7 @@ static int layer_train_step(Layer &L, const T *x, const T *y, long B, long h) {
 template <typename T>
 static int layer_mask_replaced(Layer &L, const uint8_t *mask) {
   L.w_masked = false;
+  L.w_unchecked = true;
   std::vector<long> count((size_t)L.H, 0);
   for (long i = 0; i < L.N; i++)
     for (long h = 0; h < L.H; h++) count[(size_t)h] += mask[i * L.H + h] != 0;
@@ -351,7 +375,7 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
     const long B = (lo + maxB <= Ns) ? maxB : Ns - lo;
     const T *x = (const T *)net->Xp + lo * net->NF;
     for (int l = 0; l < layer; l++) {
-      if ((rc = layer_forward<T>(net->layers[l], x, B))) return rc;
+      if ((rc = layer_forward<T>(net, net->layers[l], x, B))) return rc;
       x = (const T *)net->layers[l].act;
     }
     long h = -1;
@@ -368,7 +392,7 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
       // (_cpu_base_backend.py:290-295, 304-306); it has no effect on any state
       rc = layer_train_step<T>(target, x, (const T *)net->Yp + lo * net->NC, B, -1);
     } else {
-      if ((rc = layer_forward<T>(target, x, B))) return rc;
+      if ((rc = layer_forward<T>(net, target, x, B))) return rc;
       rc = layer_train_step<T>(target, x, (const T *)target.act, B, h);
     }
     if (rc) return rc;
@@ -390,7 +414,7 @@ static int net_forward_batches(sb_net *net, const void *h_images, const void *h_
   SB_REQUIRE(net->layers[0].N == NF, "image width does not match the first layer");
   for (int l = 1; l <= last_layer; l++)
     SB_REQUIRE(net->layers[l].N == net->layers[l - 1].M, "layer widths do not chain");
-  const Layer &out = net->layers[last_layer];
+  Layer &out = net->layers[last_layer];
   SB_REQUIRE(!h_labels || NC == out.M, "label width does not match the last layer");
   if (n == 0) return 0;
   int rc = ensure_act(net, maxB < n ? maxB : n);
@@ -420,7 +444,7 @@ static int net_forward_batches(sb_net *net, const void *h_images, const void *h_
       const long B = (lo + maxB <= rows) ? maxB : rows - lo;
       const T *x = (const T *)dX + lo * NF;
       for (int l = 0; l <= last_layer && !rc; l++) {
-        rc = layer_forward<T>(net->layers[l], x, B);
+        rc = layer_forward<T>(net, net->layers[l], x, B);
         x = (const T *)net->layers[l].act;
       }
       if (rc) break;
@@ -657,6 +681,7 @@ int sb_net_create(sb_net **net, int dtype) {
   n->dtype = dtype;
   n->esize = dtype == SB_F32 ? 4 : 8;
   hipError_t e = hipMalloc((void **)&n->d_correct, sizeof(unsigned long long));
+  if (e == hipSuccess) e = hipMalloc((void **)&n->d_unmasked, sizeof(unsigned long long));
   if (e == hipSuccess) e = hipEventCreateWithFlags(&n->perm_copied, hipEventDisableTiming);
   if (e != hipSuccess) {
     delete n;
@@ -687,6 +712,7 @@ int sb_net_destroy(sb_net *net) {
   int rc = sb_net_training_done(net);
   for (auto &L : net->layers) rc |= layer_free(L);
   if (net->d_correct) SB_HIP(hipFree(net->d_correct));
+  if (net->d_unmasked) SB_HIP(hipFree(net->d_unmasked));
   if (net->perm_copied) SB_HIP(hipEventDestroy(net->perm_copied));
   delete net;
   return rc;
@@ -735,7 +761,7 @@ int sb_net_set_layer_state(sb_net *net, int layer, const char *name, const void 
   rc = sb_memcpy_h2d(s.ptr, h_src, bytes);
   if (rc) return rc;
   Layer &L = net->layers[layer];
-  if (s.ptr == L.W) L.w_masked = false;
+  if (s.ptr == L.W) L.w_masked = false, L.w_unchecked = true;
   if (s.ptr == L.wmask)
     return net->dtype == SB_F32 ? layer_mask_replaced<float>(L, (const uint8_t *)h_src)
                                 : layer_mask_replaced<double>(L, (const uint8_t *)h_src);

@@ -286,7 +286,10 @@ def test_forward_over_connected_rows_tracks_the_state(hb, dtype, tol):
     W, b, mask = layer.weights, layer.bias, layer.wmask
     assert np.all(W[np.repeat(mask, 20, axis=1) == 0] == 0)
     assert rel_err(net.forward(xt, last_layer=0), dense(W, b)) <= 4 * tol  # row lists (after rewiring)
-    # an unmasked W written from outside must be used as it is
+    # a masked W written from outside (a restored checkpoint) is recognised as such ...
+    layer.weights = W
+    assert rel_err(net.forward(xt, last_layer=0), dense(W, b)) <= 4 * tol
+    # ... and an unmasked one must be used as it is
     W2 = (W + 0.01).astype(dtype)
     layer.weights = W2
     assert rel_err(net.forward(xt, last_layer=0), dense(W2, b)) <= 4 * tol
