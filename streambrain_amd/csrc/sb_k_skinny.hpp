@@ -13,9 +13,14 @@ namespace sb {
 // act[b, :] = softmax_per_hypercolumn(x[b, :] . W + bias)      omp.cc:70-87 + kernels_numpy.py:13-25
 // One workgroup per batch row.  Partial sums over the rows r, r + R, ... are added up in the order of r
 // (fixed, so the result is deterministic).
+// Classification in the same launch (_cpu_base_backend.py:239-241), when pred or labels is given: the
+// row's first maximal unit goes to pred[b], and *correct counts the rows whose first maximal unit is the
+// labels' first maximal unit -- the result k_argmax_rows gives on the stored activations.
 template <typename T>
 __global__ __launch_bounds__(256) void k_forward_skinny(T *act, const T *x, const T *W, const T *bias,
-                                                        long N, long M, long Mc, int softmax) {
+                                                        long N, long M, long Mc, int softmax,
+                                                        const T *labels, int32_t *pred,
+                                                        unsigned long long *correct) {
   __shared__ T part[256];
   __shared__ T logit[32];
   const int tid = threadIdx.x;
@@ -48,8 +53,9 @@ __global__ __launch_bounds__(256) void k_forward_skinny(T *act, const T *x, cons
     logit[tid] = s + bias[tid];
   }
   __syncthreads();
+  T v = T(0);
   if (tid < M) {
-    T v = logit[tid];
+    v = logit[tid];
     if (softmax) {
       const int h0 = (tid / (int)Mc) * (int)Mc;  // first unit of this thread's hypercolumn
       T mx = -INFINITY;
@@ -59,6 +65,21 @@ __global__ __launch_bounds__(256) void k_forward_skinny(T *act, const T *x, cons
       v = Real<T>::exp_(v - mx) / sum;
     }
     act[(long)blockIdx.x * M + tid] = v;
+  }
+  if (pred == nullptr && labels == nullptr) return;  // uniform
+  __syncthreads();  // everybody has read the logits
+  if (tid < M) logit[tid] = v;
+  __syncthreads();
+  if (tid == 0) {
+    int best = 0;
+    for (int c = 1; c < M; c++) best = logit[c] > logit[best] ? c : best;
+    if (pred) pred[blockIdx.x] = best;
+    if (labels) {
+      const T *lab = labels + (long)blockIdx.x * M;
+      int lbest = 0;
+      for (int c = 1; c < M; c++) lbest = lab[c] > lab[lbest] ? c : lbest;
+      if (lbest == best) atomicAdd(correct, 1ull);
+    }
   }
 }
 

@@ -61,6 +61,12 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
 template <typename T>
 int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias, long B, long N,
                    long H, long Mc, bool softmax);
+// The same followed by launch_argmax_rows on the result (pred and / or labels + correct given); layers of
+// at most 32 units do both in one launch.
+template <typename T>
+int launch_forward_classify(hipStream_t st, T *act, const T *x, const T *W, const T *bias, long B, long N,
+                            long H, long Mc, bool softmax, const T *labels, int32_t *pred,
+                            unsigned long long *correct);
 // The same result for a layer whose W is zero wherever wmask is 0, from the per-hypercolumn lists of
 // connected rows that launch_mask_rows builds (rows: [H, cap] ascending indices, the rest -1; cap a
 // multiple of 16; row_cnt: [H]); forward_rows_supported says whether the kernel takes the shape.

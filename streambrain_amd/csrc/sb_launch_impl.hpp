@@ -50,6 +50,13 @@ static inline int device_cu_count() {
 template <typename T>
 int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias, long B, long N,
                    long H, long Mc, bool softmax) {
+  return launch_forward_classify<T>(st, act, x, W, bias, B, N, H, Mc, softmax, nullptr, nullptr, nullptr);
+}
+
+template <typename T>
+int launch_forward_classify(hipStream_t st, T *act, const T *x, const T *W, const T *bias, long B, long N,
+                            long H, long Mc, bool softmax, const T *labels, int32_t *pred,
+                            unsigned long long *correct) {
   constexpr int VW = Real<T>::VW;
   constexpr int GW = 16 * VW;
   SB_REQUIRE(act && x && W && bias, "null pointer");
@@ -59,10 +66,16 @@ int launch_forward(hipStream_t st, T *act, const T *x, const T *W, const T *bias
   if (M <= 32) {  // a handful of output units: plain vector arithmetic, one workgroup per batch row
     SB_REQUIRE(B < (1L << 31), "batch too large for one launch");
     ProfScope prof_(st, K_FORWARD);
+    SB_REQUIRE(!labels || correct, "labels need a counter");
     hipLaunchKernelGGL((k_forward_skinny<T>), dim3((unsigned)B), dim3(256), 0, st, act, x, W, bias, N, M, Mc,
-                       softmax ? 1 : 0);
+                       softmax ? 1 : 0, labels, pred, correct);
     SB_LAUNCH_CHECK();
     return 0;
+  }
+  if (labels || pred) {  // wider layers: the forward pass, then the classification kernel
+    int rc = launch_forward<T>(st, act, x, W, bias, B, N, H, Mc, softmax);
+    if (rc) return rc;
+    return launch_argmax_rows<T>(st, act, labels, B, M, pred, correct);
   }
   // per-lane byte offsets inside one chunk of 16 rows of x or W are 32-bit
   SB_REQUIRE(16 * (N > M ? N : M) * (long)sizeof(T) < (1L << 31), "layer too wide for the forward kernel");
@@ -347,6 +360,9 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
 #define SB_INSTANTIATE_LAUNCHERS(T)                                                                   \
   template int launch_forward<T>(hipStream_t, T *, const T *, const T *, const T *, long, long, long, \
                                  long, bool);                                                         \
+  template int launch_forward_classify<T>(hipStream_t, T *, const T *, const T *, const T *, long,    \
+                                          long, long, long, bool, const T *, int32_t *,               \
+                                          unsigned long long *);                                      \
   template bool forward_rows_supported<T>(const T *, long, long, long);                               \
   template int launch_forward_rows<T>(hipStream_t, T *, const T *, const T *, const T *, const int *, \
                                       const int *, long, long, long, long, long);                     \

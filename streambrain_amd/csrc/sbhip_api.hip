@@ -443,12 +443,20 @@ static int net_forward_batches(sb_net *net, const void *h_images, const void *h_
     for (long lo = 0; lo < rows && !rc; lo += maxB) {
       const long B = (lo + maxB <= rows) ? maxB : rows - lo;
       const T *x = (const T *)dX + lo * NF;
+      const bool classify = h_labels || h_pred;
       for (int l = 0; l <= last_layer && !rc; l++) {
-        rc = layer_forward<T>(net, net->layers[l], x, B);
-        x = (const T *)net->layers[l].act;
+        Layer &L = net->layers[l];
+        if (l == last_layer && classify && !L.plastic)
+          // output layer: activation and classification (first maximal unit, comparison with the labels)
+          rc = launch_forward_classify<T>(st, (T *)L.act, x, (const T *)L.W, (const T *)L.bias, B, L.N, L.H,
+                                          L.Mc, true, h_labels ? (const T *)dY + lo * NC : nullptr,
+                                          dP ? dP + lo : nullptr, net->d_correct);
+        else
+          rc = layer_forward<T>(net, L, x, B);
+        x = (const T *)L.act;
       }
       if (rc) break;
-      if (h_labels || h_pred)
+      if (classify && out.plastic)
         rc = launch_argmax_rows<T>(st, (const T *)out.act, h_labels ? (const T *)dY + lo * NC : nullptr,
                                    B, out.M, dP ? dP + lo : nullptr, net->d_correct);
       if (!rc && h_act)
