@@ -98,19 +98,19 @@ __global__ __launch_bounds__(256) void k_train_skinny(TrainArgs<T> a) {
   if (r >= R || i >= a.N) return;  // no barriers below
   T dot = T(0), sx = T(0), sy = T(0);
   const T *xp = a.x + i, *yp = a.y + j;
-  // 16 batch rows of loads in flight (branch-free: past the batch the last row is re-read and counts
+  // 32 batch rows of loads in flight (branch-free: past the batch the last row is re-read and counts
   // as 0), then the ordered arithmetic; the pointers advance by one row per load
-  for (long b0 = 0; b0 < a.B; b0 += 16) {
-    T xv[16], yv[16];
+  for (long b0 = 0; b0 < a.B; b0 += 32) {
+    T xv[32], yv[32];
 #pragma unroll
-    for (int k = 0; k < 16; k++) {
+    for (int k = 0; k < 32; k++) {
       const bool live = b0 + k < a.B;  // uniform; the pointers stop at the last row of the batch
       xv[k] = *xp, yv[k] = *yp;
       xp += live && b0 + k + 1 < a.B ? a.N : 0;
       yp += live && b0 + k + 1 < a.B ? a.M : 0;
     }
 #pragma unroll
-    for (int k = 0; k < 16; k++) {
+    for (int k = 0; k < 32; k++) {
       const bool live = b0 + k < a.B;
       const T xk = live ? xv[k] : T(0), yk = live ? yv[k] : T(0);
       dot += xk * yk;
