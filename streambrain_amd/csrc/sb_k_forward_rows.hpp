@@ -4,8 +4,9 @@
 // wherever wmask[i, h] is 0, so in  act = softmax_per_hypercolumn(x . W + bias)  (omp.cc:70-87 +
 // kernels_numpy.py:13-25) those rows add exact zeros to hypercolumn h.  With a connection density of
 // 0.1 nine tenths of the reduction are such zeros.  k_forward_rows skips them: per hypercolumn it walks
-// the ascending list of connected rows (k_mask_rows in sb_kernels.hpp keeps the lists in step with wmask) and gathers
-// those rows of W and those columns of x.  Same tiling, accumulator layout and epilogue as k_forward.
+// the ascending list of connected rows (k_mask_rows in sb_kernels.hpp keeps the lists in step with
+// wmask) and gathers those rows of W and those columns of x.  Same tiling, accumulator layout and
+// epilogue as k_forward.
 #pragma once
 #include "sb_k_forward.hpp"
 #include "sb_kernels.hpp"
@@ -25,7 +26,8 @@ struct ForwardRowsArgs {
 // of 4*VW entries.  Per chunk, lane (p,q) reads the VW list entries VW*q .. VW*q+VW-1 from LDS, then
 // x[b0+p, row] for each of them (the A operands of VW MFMA steps) and VW*NG vectors of VW columns of
 // W[row, :] (the B operands); the operands of one chunk are in flight while the previous one is
-// multiplied.  A padding entry (-1) contributes x = 0 times row 0 of W.  Nothing up to the first MFMAs
+// multiplied.  A padding entry (-1) contributes x = 0 times row 0 of W (which under the kernel's
+// precondition is either zero for this hypercolumn or a term of the sum anyway).  Nothing up to the first MFMAs
 // depends on the hypercolumn's row count: every wavefront multiplies its first chunk of the first
 // segment, which is padding where the list is shorter.
 // Requires M % VW == 0, Mc % VW == 0 and 16-byte aligned W.

@@ -172,7 +172,8 @@ __device__ __forceinline__ KeyIdx<uint32_t> wave_pick(KeyIdx<uint32_t> c) {
   v = larger(v, dpp_move_k<kDppSwap2>(v));
   v = larger(v, dpp_move_k<kDppHalfMirror>(v));
   v = larger(v, dpp_move_k<kDppMirror>(v));
-  const uint64_t m = larger(larger(readlane_k(v, 0), readlane_k(v, 16)), larger(readlane_k(v, 32), readlane_k(v, 48)));
+  const uint64_t m = larger(larger(readlane_k(v, 0), readlane_k(v, 16)),
+                            larger(readlane_k(v, 32), readlane_k(v, 48)));
   return KeyIdx<uint32_t>{(uint32_t)(m >> 32), (int)(uint32_t)m - 1};
 }
 

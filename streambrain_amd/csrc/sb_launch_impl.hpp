@@ -180,7 +180,8 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   const TraceScalars<T> s = TraceScalars<T>::from(taupdt, cthr);
   TrainArgs<T> a;
   a.x = x; a.y = y; a.Cij = Cij; a.W = W; a.Ci = Ci; a.Cj = Cj; a.Ci_next = Ci_next; a.Cj_next = Cj_next;
-  a.wmask = wmask; a.w_masked = (wmask && w_masked) ? 1 : 0; a.bias_mode = bias_mode; a.bias = bias; a.kbi = kbi;
+  a.wmask = wmask; a.w_masked = (wmask && w_masked) ? 1 : 0;
+  a.bias_mode = bias_mode; a.bias = bias; a.kbi = kbi;
   a.B = B; a.N = N; a.M = M; a.H = H; a.Mc = Mc;
   a.tau = s.tau; a.omt = s.omt; a.fB = (T)B; a.invB = (T)1 / (T)B; a.cthr = s.cthr; a.cthr4 = s.cthr4;
   a.khalf = khalf; a.pmin = pmin; a.taubdt = taubdt;
@@ -286,8 +287,8 @@ int launch_mask_fix_weights(hipStream_t st, T *W, const uint8_t *wmask, const T 
   const TraceScalars<T> s = TraceScalars<T>::from(T(0), cthr);
   ProfScope prof_(st, K_MASK_FIX);
   // with a row list, one more workgroup rebuilds the list of hypercolumn h
-  hipLaunchKernelGGL((k_mask_fix_weights<T>), dim3((unsigned)(cdiv(N * Mc, 256) + (rows ? 1 : 0))), dim3(256), 0,
-                     st, W, wmask, Ci, Cj, Cij, cthr, s.cthr4, N, H * Mc, H, Mc, h, rows, row_cnt, cap);
+  const long blocks = cdiv(N * Mc, 256) + (rows ? 1 : 0);
+  hipLaunchKernelGGL((k_mask_fix_weights<T>), dim3((unsigned)blocks), dim3(256), 0, st, W, wmask, Ci, Cj, Cij, cthr, s.cthr4, N, H * Mc, H, Mc, h, rows, row_cnt, cap);
   SB_LAUNCH_CHECK();
   return 0;
 }

@@ -285,7 +285,8 @@ static int layer_train_step(Layer &L, const T *x, const T *y, long B, long h) {
   if (rc) return rc;
   std::swap(L.Ci, L.Ci_alt);
   std::swap(L.Cj, L.Cj_alt);
-  if (L.plastic) L.w_masked = true, L.w_unchecked = false;  // every entry of W has just been written under the mask
+  // every entry of W has just been written under the mask
+  if (L.plastic) L.w_masked = true, L.w_unchecked = false;
   if (L.plastic && h >= 0) {
     rc = launch_update_mask<T>(st, L.wmask, (const T *)nullptr, (const T *)L.Ci, (const T *)L.Cj,
                                (const T *)L.Cij, cthr, L.N, L.H, L.Mc, h, 16, (T *)L.nom, L.csum);
