@@ -288,7 +288,8 @@ int launch_mask_fix_weights(hipStream_t st, T *W, const uint8_t *wmask, const T 
   ProfScope prof_(st, K_MASK_FIX);
   // with a row list, one more workgroup rebuilds the list of hypercolumn h
   const long blocks = cdiv(N * Mc, 256) + (rows ? 1 : 0);
-  hipLaunchKernelGGL((k_mask_fix_weights<T>), dim3((unsigned)blocks), dim3(256), 0, st, W, wmask, Ci, Cj, Cij, cthr, s.cthr4, N, H * Mc, H, Mc, h, rows, row_cnt, cap);
+  hipLaunchKernelGGL((k_mask_fix_weights<T>), dim3((unsigned)blocks), dim3(256), 0, st, W, wmask, Ci, Cj, Cij,
+                     cthr, s.cthr4, N, H * Mc, H, Mc, h, rows, row_cnt, cap);
   SB_LAUNCH_CHECK();
   return 0;
 }
