@@ -185,7 +185,11 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
 // 8: with LW = 3 the last group's lanes load LW consecutive columns (12 bytes) instead of VW, and a
 // quarter of that group's MFMAs disappears.  The launcher picks LW < VW only when no vector of the last
 // group straddles the end of the tile.
-template <typename T, int NG, bool FUSE, bool VEC, int NWAVES, int LW = Real<T>::VW>
+//
+// RB: row blocks per workgroup.  The tile is 16*RB batch rows, every W vector a lane loads feeds RB MFMAs
+// instead of one, and W crosses the L2 -> L1 path 1/RB as often: for batches of many rows, where that path
+// is what bounds the kernel.  The epilogue handles the row blocks one after the other.
+template <typename T, int NG, bool FUSE, bool VEC, int NWAVES, int LW = Real<T>::VW, int RB = 1>
 __global__ __launch_bounds__(64 * NWAVES) __attribute__((amdgpu_waves_per_eu(NWAVES / 4, NWAVES / 4)))
 void k_forward(ForwardArgs<T> a) {
   constexpr int VW = Real<T>::VW;
@@ -208,35 +212,42 @@ void k_forward(ForwardArgs<T> a) {
 
   const int tid = threadIdx.x, lane = tid & 63, p = lane & 15, q = lane >> 4;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, in a scalar register: uniform branches
-  const long b0 = bt * 16;
+  const long b0 = bt * (16 * RB);
   const long j0 = FUSE ? ct * a.Mc : ct * (NG * GW);
   const long jend = FUSE ? j0 + a.Mc : (j0 + NG * GW < a.M ? j0 + NG * GW : a.M);
-  const bool row_ok = (b0 + p) < a.B;
-  const T *xrow = a.x + (b0 + p) * a.N;
 
-  acc_t acc[NG][VW];
+  acc_t acc[RB][NG][VW];
 #pragma unroll
-  for (int g = 0; g < NG; g++)
+  for (int r = 0; r < RB; r++)
 #pragma unroll
-    for (int c = 0; c < VW; c++) acc[g][c] = acc_t{0, 0, 0, 0};
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+      for (int c = 0; c < VW; c++) acc[r][g][c] = acc_t{0, 0, 0, 0};
 
   // ring of D chunk buffers: D-1 chunks of loads are in flight while one is being multiplied
   constexpr int D = 2;  // measured: deeper rings are slower, the CU cannot keep more loads in flight anyway
-  T xr[D][VW];
+  T xr[D][RB][VW];
   T wr[D][VW][NG][VW];
 
-  auto compute = [&](const T(&xi)[VW], const T(&wi)[VW][NG][VW]) {
+  auto compute = [&](const T(&xi)[RB][VW], const T(&wi)[VW][NG][VW]) {
 #pragma unroll
     for (int s = 0; s < VW; s++)
 #pragma unroll
       for (int g = 0; g < NG; g++)
 #pragma unroll
         for (int c = 0; c < VW; c++)
-          if (c < gwidth(g)) acc[g][c] = Real<T>::mfma(xi[s], wi[s][g][c], acc[g][c]);
+          if (c < gwidth(g)) {
+#pragma unroll
+            for (int r = 0; r < RB; r++) acc[r][g][c] = Real<T>::mfma(xi[r][s], wi[s][g][c], acc[r][g][c]);
+          }
   };
-  auto load_guarded = [&](long kc, T(&xo)[VW], T(&wo)[VW][NG][VW]) {
+  auto load_guarded = [&](long kc, T(&xo)[RB][VW], T(&wo)[VW][NG][VW]) {
     const long kk = kc * KC + VW * q;
-    load_vw<T, VEC>(xo, xrow, kk, a.N, row_ok);
+#pragma unroll
+    for (int r = 0; r < RB; r++) {
+      const long row = b0 + 16 * r + p;
+      load_vw<T, VEC>(xo[r], a.x + (row < a.B ? row : 0) * a.N, kk, a.N, row < a.B);
+    }
 #pragma unroll
     for (int s = 0; s < VW; s++) {
       const long krow = kk + s;
@@ -272,7 +283,9 @@ void k_forward(ForwardArgs<T> a) {
     const T *wbase = a.W + (long)w * KC * a.M + j0;             // uniform
     long xleft = (a.B - b0) * a.N - (long)w * KC;               // elements from xbase to the end of x
     long wleft = (a.N - (long)w * KC) * a.M - j0;               // ... of W
-    const unsigned xat = (unsigned)(((long)p * a.N + VW * q) * ES);
+    unsigned xat[RB];
+#pragma unroll
+    for (int r = 0; r < RB; r++) xat[r] = (unsigned)(((long)(16 * r + p) * a.N + VW * q) * ES);
     unsigned wat[VW][NG];
 #pragma unroll
     for (int s = 0; s < VW; s++)
@@ -286,9 +299,10 @@ void k_forward(ForwardArgs<T> a) {
     // past the last chunk reads whatever lies there (or zeros past the arrays) and is never used, so
     // the compiler can keep exact wait counts and D-1 chunks really are in flight.
     const long n = w < nfull ? (nfull - 1 - w) / NWAVES + 1 : 0;
-    auto load_next = [&](T(&xo)[VW], T(&wo)[VW][NG][VW]) {
+    auto load_next = [&](T(&xo)[RB][VW], T(&wo)[VW][NG][VW]) {
       const BufferWindow<T> xwin(xbase, xleft), wwin(wbase, wleft);
-      xwin.template load_n<VW>(xo, xat);
+#pragma unroll
+      for (int r = 0; r < RB; r++) xwin.template load_n<VW>(xo[r], xat[r]);
 #pragma unroll
       for (int s = 0; s < VW; s++)
 #pragma unroll
@@ -339,7 +353,11 @@ void k_forward(ForwardArgs<T> a) {
   }
 
   SB_PHASE_MARK(1);
-  forward_finish<T, NG, FUSE, NWAVES, LW>(acc, bv, red, a.act, a.B, a.M, b0, j0, ncol);
+#pragma unroll
+  for (int r = 0; r < RB; r++) {
+    if (r > 0) __syncthreads();  // the previous row block's sums have been read
+    forward_finish<T, NG, FUSE, NWAVES, LW>(acc[r], bv, red, a.act, a.B, a.M, b0 + 16 * r, j0, ncol);
+  }
   SB_PHASE_MARK(3);
 }
 

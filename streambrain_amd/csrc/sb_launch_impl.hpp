@@ -93,10 +93,26 @@ int launch_forward_classify(hipStream_t st, T *act, const T *x, const T *W, cons
     if (vec && nblocks == 7) {
       constexpr int NGL = 8 / VW, LWL = 7 - (NGL - 1) * VW;  // float: 2 groups, 3 blocks; double: 4, 1
       if ((Mc - (NGL - 1) * GW) % LWL == 0) {
+        // Large batches: 64 or 32 rows per workgroup instead of 16 while there still are enough tiles for
+        // eight / four rounds of workgroups, so that W crosses the L2 -> L1 path a quarter / half as often.
+        const long cus = device_cu_count();
+        // (double: at most 32 rows, 64 do not fit the register file)
+        const long rb = sizeof(T) == 4 && H * cdiv(B, 64) >= 8 * cus ? 4 : (H * cdiv(B, 32) >= 4 * cus ? 2 : 1);
+        a.batch_tiles = cdiv(B, 16 * rb);
+        SB_REQUIRE(16 * rb * N * (long)sizeof(T) < (1L << 31), "layer too wide for the forward kernel");
         ProfScope prof_(st, K_FORWARD);
         const long grid = 8 * cdiv(a.col_tiles * a.batch_tiles, 8);
         SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
-        hipLaunchKernelGGL((k_forward<T, NGL, true, true, 8, LWL>), dim3((unsigned)grid), dim3(512), 0, st, a);
+        if constexpr (sizeof(T) == 4) {
+          if (rb == 4)
+            hipLaunchKernelGGL((k_forward<T, NGL, true, true, 8, LWL, 4>), dim3((unsigned)grid), dim3(512), 0, st,
+                               a);
+        }
+        if (rb == 4) {
+        } else if (rb == 2)
+          hipLaunchKernelGGL((k_forward<T, NGL, true, true, 8, LWL, 2>), dim3((unsigned)grid), dim3(512), 0, st, a);
+        else
+          hipLaunchKernelGGL((k_forward<T, NGL, true, true, 8, LWL>), dim3((unsigned)grid), dim3(512), 0, st, a);
         SB_LAUNCH_CHECK();
         return 0;
       }

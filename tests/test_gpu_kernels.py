@@ -111,7 +111,9 @@ def test_softmax_minicolumns(k, oracle, dtype, B, H, Mc):
 @pytest.mark.parametrize("B,N,H,Mc", [(1, 1, 1, 1), (7, 13, 3, 5), (128, 1568, 30, 100),
                                       (96, 1568, 30, 100), (33, 300, 2, 200), (20, 100, 2, 256),
                                       (16, 64, 2, 300), (40, 3000, 1, 10), (10, 50, 3, 66),
-                                      (12, 40, 2, 224)])
+                                      (12, 40, 2, 224),
+                                      # many tiles: 32 and 64 batch rows per workgroup, ragged last tile
+                                      (1000, 44, 32, 100), (2030, 36, 64, 100)])
 def test_compute_activation_fused(k, oracle, dtype, B, N, H, Mc):
     rng = np.random.default_rng(B + N + H + Mc)
     M = H * Mc
