@@ -31,7 +31,8 @@ struct ForwardRowsArgs {
 // depends on the hypercolumn's row count: every wavefront multiplies its first chunk of the first
 // segment, which is padding where the list is shorter.
 // Requires M % VW == 0, Mc % VW == 0 and 16-byte aligned W.
-template <typename T, int NG, int NWAVES>
+// RB: row blocks per workgroup, as in k_forward: 16*RB batch rows share every gathered W vector.
+template <typename T, int NG, int NWAVES, int RB = 1>
 __global__ __launch_bounds__(64 * NWAVES)
 __attribute__((amdgpu_waves_per_eu(NWAVES >= 4 ? NWAVES / 4 : 1, NWAVES >= 4 ? NWAVES / 4 : 1)))
 void k_forward_rows(ForwardRowsArgs<T> ar) {
@@ -57,7 +58,7 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
 
   const int tid = threadIdx.x, lane = tid & 63, p = lane & 15, q = lane >> 4;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const long b0 = bt * 16;
+  const long b0 = bt * (16 * RB);
   const long j0 = ct * a.Mc;
   const long ncol = a.Mc;
   const int *list = ar.rows + ct * ar.cap;
@@ -83,36 +84,44 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
   request_segment(0);
   const int cnt = ar.row_cnt[ct];
 
-  acc_t acc[NG][VW];
+  acc_t acc[RB][NG][VW];
 #pragma unroll
-  for (int g = 0; g < NG; g++)
+  for (int r = 0; r < RB; r++)
 #pragma unroll
-    for (int c = 0; c < VW; c++) acc[g][c] = acc_t{0, 0, 0, 0};
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+      for (int c = 0; c < VW; c++) acc[r][g][c] = acc_t{0, 0, 0, 0};
 
   T bv[ForwardBias<T, NG, NWAVES>::PT];
   ForwardBias<T, NG, NWAVES>::load(bv, a.bias, j0, ncol);
 
-  // x through a bounds-checked window over this tile's 16 batch rows: rows past the batch and padding
+  // x through a bounds-checked window over this tile's batch rows: rows past the batch and padding
   // entries (offset kOutside) read zero
   const BufferWindow<T> xwin(a.x + b0 * a.N, (a.B - b0) * a.N);
-  const unsigned xat = (unsigned)((long)p * a.N * sizeof(T));
+  unsigned xat[RB];
+#pragma unroll
+  for (int r = 0; r < RB; r++) xat[r] = (unsigned)((long)(16 * r + p) * a.N * sizeof(T));
   // W: this lane's columns of group g, or the tile's first columns where the group hangs over the end
   // of the hypercolumn (those accumulator columns are never stored)
   const T *wcol[NG];
 #pragma unroll
   for (int g = 0; g < NG; g++) wcol[g] = a.W + j0 + (TC::gcol(g, p) < ncol ? TC::gcol(g, p) : 0);
 
-  T xr[2][VW];
+  T xr[2][RB][VW];
   T wr[2][VW][NG][VW];
   // operands of chunk c of the staged segment (c past the segment: its last chunk again, never used)
-  auto request = [&](int c, T(&xo)[VW], T(&wo)[VW][NG][VW]) {
+  auto request = [&](int c, T(&xo)[RB][VW], T(&wo)[VW][NG][VW]) {
     const ivec_t idx = *reinterpret_cast<const ivec_t *>(&sidx[(c < SEGC ? c : SEGC - 1) * KC + VW * q]);
 #pragma unroll
     for (int s = 0; s < VW; s++) {
       const int r = idx[s];
-      T one[1];
-      xwin.template load_n<1>(one, r < 0 ? BufferWindow<T>::kOutside : xat + (unsigned)r * (unsigned)sizeof(T));
-      xo[s] = one[0];
+#pragma unroll
+      for (int rb = 0; rb < RB; rb++) {
+        T one[1];
+        xwin.template load_n<1>(one, r < 0 ? BufferWindow<T>::kOutside
+                                           : xat[rb] + (unsigned)r * (unsigned)sizeof(T));
+        xo[rb][s] = one[0];
+      }
       const long roff = (long)(r < 0 ? 0 : r) * a.M;
 #pragma unroll
       for (int g = 0; g < NG; g++) {
@@ -122,13 +131,15 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
       }
     }
   };
-  auto compute = [&](const T(&xi)[VW], const T(&wi)[VW][NG][VW]) {
+  auto compute = [&](const T(&xi)[RB][VW], const T(&wi)[VW][NG][VW]) {
 #pragma unroll
     for (int s = 0; s < VW; s++)
 #pragma unroll
       for (int g = 0; g < NG; g++)
 #pragma unroll
-        for (int c = 0; c < VW; c++) acc[g][c] = Real<T>::mfma(xi[s], wi[s][g][c], acc[g][c]);
+        for (int c = 0; c < VW; c++)
+#pragma unroll
+          for (int r = 0; r < RB; r++) acc[r][g][c] = Real<T>::mfma(xi[r][s], wi[s][g][c], acc[r][g][c]);
   };
 
   for (long seg0 = 0;;) {
@@ -166,7 +177,11 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
     __syncthreads();  // everyone is done with the staged segment
   }
   SB_PHASE_MARK(1);
-  forward_finish<T, NG, true, NWAVES, VW>(acc, bv, red, a.act, a.B, a.M, b0, j0, ncol);
+#pragma unroll
+  for (int r = 0; r < RB; r++) {
+    if (r > 0) __syncthreads();  // the previous row block's sums have been read
+    forward_finish<T, NG, true, NWAVES, VW>(acc[r], bv, red, a.act, a.B, a.M, b0 + 16 * r, j0, ncol);
+  }
   SB_PHASE_MARK(3);
 }
 

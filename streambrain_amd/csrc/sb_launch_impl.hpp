@@ -139,13 +139,27 @@ bool forward_rows_supported(const T *W, long N, long H, long Mc) {
 }
 
 template <typename T, int NG>
-static int forward_rows_variant(hipStream_t st, const ForwardRowsArgs<T> &a) {
+static int forward_rows_variant(hipStream_t st, ForwardRowsArgs<T> a) {
   ProfScope prof_(st, K_FORWARD);
-  const long grid = 8 * cdiv(a.f.col_tiles * a.f.batch_tiles, 8);
-  SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
   // four wavefronts measured best (8: 8.8 us, 4: 8.2 us, 2: 9.9 us, 16: 10.7 us at 1568 -> 30x100, density 0.1)
   constexpr int NW = 4;
-  hipLaunchKernelGGL((k_forward_rows<T, NG, NW>), dim3((unsigned)grid), dim3(64 * NW), 0, st, a);
+  // large batches: 64 or 32 rows per workgroup while there are tiles for eight / four rounds of
+  // workgroups (as in launch_forward; double and wide hypercolumns: at most 32 rows, for registers)
+  const long cus = device_cu_count(), H = a.f.col_tiles, B = a.f.B;
+  constexpr bool fits4 = sizeof(T) == 4 && NG <= 2;
+  const long rb = fits4 && H * cdiv(B, 64) >= 8 * cus ? 4 : (H * cdiv(B, 32) >= 4 * cus ? 2 : 1);
+  a.f.batch_tiles = cdiv(B, 16 * rb);
+  SB_REQUIRE(16 * rb * a.f.N * (long)sizeof(T) < (1L << 31), "layer too wide for the forward kernel");
+  const long grid = 8 * cdiv(a.f.col_tiles * a.f.batch_tiles, 8);
+  SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
+  if constexpr (fits4) {
+    if (rb == 4) hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 4>), dim3((unsigned)grid), dim3(64 * NW), 0, st, a);
+  }
+  if (rb == 4) {
+  } else if (rb == 2)
+    hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 2>), dim3((unsigned)grid), dim3(64 * NW), 0, st, a);
+  else
+    hipLaunchKernelGGL((k_forward_rows<T, NG, NW>), dim3((unsigned)grid), dim3(64 * NW), 0, st, a);
   SB_LAUNCH_CHECK();
   return 0;
 }

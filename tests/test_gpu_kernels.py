@@ -72,6 +72,8 @@ def test_mask_rows(k, N, H, density):
                                               (16, 64, 2, 64, 1.0), (20, 100, 2, 256, 0.05),
                                               (5, 50, 3, 12, 0.0), (300, 5000, 4, 100, 0.4),
                                               (20, 6000, 2, 64, 0.5),  # lists longer than one LDS segment
+                                              # many tiles: 32 and 64 batch rows per workgroup, ragged
+                                              (1000, 300, 32, 100, 0.2), (2030, 200, 64, 100, 0.3),
                                               (12, 40, 2, 224, 0.5)])
 def test_compute_activation_rows(k, oracle, dtype, B, N, H, Mc, density):
     """The row-list forward kernel against the dense reference computation on the masked weights."""
