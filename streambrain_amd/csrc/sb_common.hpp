@@ -184,6 +184,37 @@ struct BufferWindow {
   }
 };
 
+// Exchange inside a row of 16 lanes with data-parallel-primitive moves (no LDS round trip).  The four
+// controls below -- swap neighbours, swap pairs, mirror each half row, mirror the row -- applied in
+// turn with a commutative pick leave the row-wide result in every one of the 16 lanes.
+constexpr int kDppSwap1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppSwap2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // row_half_mirror
+constexpr int kDppMirror = 0x140;      // row_mirror
+template <int CTRL>
+__device__ __forceinline__ int dpp_move(int v) {
+  return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xF, 0xF, false);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(dpp_move<CTRL>(__float_as_int(v)));
+}
+template <int CTRL>
+__device__ __forceinline__ double dpp_move(double v) {
+  const long long b = __double_as_longlong(v);
+  const int lo = dpp_move<CTRL>((int)(b & 0xffffffffLL)), hi = dpp_move<CTRL>((int)(b >> 32));
+  return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+// op-reduction over each row of 16 lanes; every lane of the row ends with the result
+template <typename T, typename Op>
+__device__ __forceinline__ T row16_reduce(T v, Op op) {
+  v = op(v, dpp_move<kDppSwap1>(v));
+  v = op(v, dpp_move<kDppSwap2>(v));
+  v = op(v, dpp_move<kDppHalfMirror>(v));
+  v = op(v, dpp_move<kDppMirror>(v));
+  return v;
+}
+
 // The weight of one synapse from its traces, shared by the trace/weight kernel and the rewiring
 // kernels so both see bit-identical values:  log(max(cij, cthr^4) / (ci * cj)) evaluated as
 // log(max(cij, cthr^4) * (1/ci) * (1/cj)).  rci / rcj are the reciprocals, or a negative number when

@@ -146,8 +146,11 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
     mx = (col < ncol && vals[t] > mx) ? vals[t] : mx;
   }
   if (FUSE) {
+    // across the TPR threads of the batch row: rows of 16 lanes by DPP moves, then across rows
+    static_assert(TPR >= 16, "at least one row of 16 lanes per batch row");
+    mx = row16_reduce(mx, [](T x_, T y_) { return y_ > x_ ? y_ : x_; });
 #pragma unroll
-    for (int o = TPR / 2; o >= 1; o >>= 1) {
+    for (int o = TPR / 2; o >= 16; o >>= 1) {
       const T other = __shfl_xor(mx, o);
       mx = other > mx ? other : mx;
     }
@@ -160,8 +163,9 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
         sum += vals[t];
       }
     }
+    sum = row16_reduce(sum, [](T x_, T y_) { return x_ + y_; });
 #pragma unroll
-    for (int o = TPR / 2; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+    for (int o = TPR / 2; o >= 16; o >>= 1) sum += __shfl_xor(sum, o);
 #pragma unroll
     for (int t = 0; t < PT; t++) vals[t] = vals[t] / sum;
   }
