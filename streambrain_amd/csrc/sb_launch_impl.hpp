@@ -97,22 +97,22 @@ int launch_forward_classify(hipStream_t st, T *act, const T *x, const T *W, cons
         // eight / four rounds of workgroups, so that W crosses the L2 -> L1 path a quarter / half as often.
         const long cus = device_cu_count();
         // (double: at most 32 rows, 64 do not fit the register file)
-        const long rb = sizeof(T) == 4 && H * cdiv(B, 64) >= 8 * cus ? 4 : (H * cdiv(B, 32) >= 4 * cus ? 2 : 1);
+        long rb = sizeof(T) == 4 && H * cdiv(B, 64) >= 8 * cus ? 4 : (H * cdiv(B, 32) >= 4 * cus ? 2 : 1);
+        // (32-bit byte offsets inside the tile's rows)
+        while (rb > 1 && 16 * rb * N * (long)sizeof(T) >= (1L << 31)) rb /= 2;
         a.batch_tiles = cdiv(B, 16 * rb);
-        SB_REQUIRE(16 * rb * N * (long)sizeof(T) < (1L << 31), "layer too wide for the forward kernel");
         ProfScope prof_(st, K_FORWARD);
         const long grid = 8 * cdiv(a.col_tiles * a.batch_tiles, 8);
         SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
+        const dim3 g((unsigned)grid);
         if constexpr (sizeof(T) == 4) {
-          if (rb == 4)
-            hipLaunchKernelGGL((k_forward<T, NGL, true, true, 8, LWL, 4>), dim3((unsigned)grid), dim3(512), 0, st,
-                               a);
+          if (rb == 4) hipLaunchKernelGGL((k_forward<T, NGL, true, true, 8, LWL, 4>), g, dim3(512), 0, st, a);
         }
         if (rb == 4) {
         } else if (rb == 2)
-          hipLaunchKernelGGL((k_forward<T, NGL, true, true, 8, LWL, 2>), dim3((unsigned)grid), dim3(512), 0, st, a);
+          hipLaunchKernelGGL((k_forward<T, NGL, true, true, 8, LWL, 2>), g, dim3(512), 0, st, a);
         else
-          hipLaunchKernelGGL((k_forward<T, NGL, true, true, 8, LWL>), dim3((unsigned)grid), dim3(512), 0, st, a);
+          hipLaunchKernelGGL((k_forward<T, NGL, true, true, 8, LWL>), g, dim3(512), 0, st, a);
         SB_LAUNCH_CHECK();
         return 0;
       }
@@ -147,9 +147,10 @@ static int forward_rows_variant(hipStream_t st, ForwardRowsArgs<T> a) {
   // workgroups (as in launch_forward; double and wide hypercolumns: at most 32 rows, for registers)
   const long cus = device_cu_count(), H = a.f.col_tiles, B = a.f.B;
   constexpr bool fits4 = sizeof(T) == 4 && NG <= 2;
-  const long rb = fits4 && H * cdiv(B, 64) >= 8 * cus ? 4 : (H * cdiv(B, 32) >= 4 * cus ? 2 : 1);
+  long rb = fits4 && H * cdiv(B, 64) >= 8 * cus ? 4 : (H * cdiv(B, 32) >= 4 * cus ? 2 : 1);
+  // (32-bit byte offsets inside the tile's rows)
+  while (rb > 1 && 16 * rb * a.f.N * (long)sizeof(T) >= (1L << 31)) rb /= 2;
   a.f.batch_tiles = cdiv(B, 16 * rb);
-  SB_REQUIRE(16 * rb * a.f.N * (long)sizeof(T) < (1L << 31), "layer too wide for the forward kernel");
   const long grid = 8 * cdiv(a.f.col_tiles * a.f.batch_tiles, 8);
   SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
   if constexpr (fits4) {
