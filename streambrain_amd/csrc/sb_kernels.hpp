@@ -84,13 +84,12 @@ __global__ __launch_bounds__(256) void k_apply_mask(T *W, const uint8_t *wmask, 
 template <typename T>
 __global__ __launch_bounds__(256) void k_count_unmasked(const T *W, const uint8_t *wmask, long N, long M,
                                                         long H, long Mc, unsigned long long *count) {
-  const long total = N * M;
-  const long stride = (long)gridDim.x * 256;
   unsigned long long mine = 0;
-  for (long e = (long)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
-    const long i = e / M;
-    const long j = e - i * M;
-    mine += (wmask[i * H + j / Mc] == 0 && !(W[e] == T(0))) ? 1 : 0;
+  for (long i = blockIdx.x; i < N; i += gridDim.x) {  // a row of W per workgroup and turn
+    const T *row = W + i * M;
+    const uint8_t *mrow = wmask + i * H;
+    for (unsigned j = threadIdx.x; j < (unsigned)M; j += 256)  // M < 2^31: 32-bit division
+      mine += (mrow[j / (unsigned)Mc] == 0 && !(row[j] == T(0))) ? 1 : 0;
   }
   if (__syncthreads_or(mine != 0) && mine != 0) atomicAdd(count, mine);
 }

@@ -344,8 +344,8 @@ int launch_count_unmasked(hipStream_t st, const T *W, const uint8_t *wmask, long
                           unsigned long long *count) {
   SB_REQUIRE(W && wmask && count, "null pointer");
   SB_REQUIRE(N > 0 && H > 0 && Mc > 0, "sizes must be positive");
-  const long total = N * H * Mc;
-  const long blocks = cdiv(total, 1024) < 8192 ? cdiv(total, 1024) : 8192;
+  SB_REQUIRE(H * Mc < (1L << 31), "dimension too large");
+  const long blocks = N < 4096 ? N : 4096;
   ProfScope prof_(st, K_APPLY_MASK);
   hipLaunchKernelGGL((k_count_unmasked<T>), dim3((unsigned)blocks), dim3(256), 0, st, W, wmask, N, H * Mc, H,
                      Mc, count);
