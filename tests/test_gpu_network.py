@@ -300,3 +300,40 @@ def test_forward_over_connected_rows_tracks_the_state(hb, dtype, tol):
     W3, mask3 = layer.weights, layer.wmask
     assert np.all(W3[np.repeat(mask3, 20, axis=1) == 0] == 0)
     assert rel_err(net.forward(xt, last_layer=0), dense(W3, layer.bias)) <= 4 * tol
+
+
+def test_full_size_epochs_keep_the_invariants_f32(hb):
+    """The headline configuration at its full size (60000 samples, 1568 -> 30 x 100, batch 128, mask
+    density 0.1), two epochs of the hidden layer, the second with rewiring -- out of the oracle's reach
+    in test time, so what is checked are the properties the update rules guarantee whatever the data:
+    the traces stay probability tables (hypercolumn sums of Cj are 1, hypercolumn sums of Cij rows are
+    Ci, everything in [0, 1]), every swap keeps the number of connections of its hypercolumn, W is zero
+    exactly where the mask is, the weights are the logarithm of the traces where it is not, and the
+    activations of a batch are per-hypercolumn distributions."""
+    rng = np.random.default_rng(1001)
+    Ns, H, Mc = 60000, 30, 100
+    X = synthetic_images(rng, Ns, 784).astype(np.float32)
+    Y = one_hot_labels(rng, Ns, 10).astype(np.float32)
+    net = build_two_layer(hb, 1568, H, Mc, 10, MNIST_HP, np.float32, seed=0)
+    layer = net._layers[0]
+    mask0 = layer.wmask.copy()
+    net.fit(X, Y, 128, [(0, 2)])
+    Ci, Cj, Cij, W, mask = layer.Ci, layer.Cj, layer.Cij, layer.weights, layer.wmask
+    assert np.isfinite(W).all() and np.isfinite(Cij).all()
+    assert Ci.min() >= 0 and Ci.max() <= 1 + 1e-5 and Cij.min() >= 0
+    assert np.allclose(Cj.reshape(H, Mc).sum(1), 1.0, atol=2e-5)
+    assert np.allclose(Cij.reshape(1568, H, Mc).sum(2), Ci[:, None], atol=2e-5)
+    # rewiring: 30 hypercolumns rewired once each in the second epoch, connection counts unchanged
+    assert np.array_equal(mask.sum(0), mask0.sum(0))
+    changed = np.flatnonzero((mask != mask0).any(0))
+    assert len(changed) >= 20 and np.all((mask != mask0).sum(0) <= 32)
+    on = np.repeat(mask, Mc, axis=1) != 0
+    assert np.all(W[~on] == 0)
+    tau = MNIST_HP["l1_taupdt"]
+    cthr = np.float32(tau / 2)
+    live = on & (Ci[:, None] >= cthr) & (Cj[None, :] >= cthr)
+    ref = np.log(np.maximum(Cij.astype(np.float64), float(cthr) ** 4) / (Ci[:, None].astype(np.float64) * Cj[None, :]))
+    assert rel_err(W[live], ref[live]) <= 2e-5
+    assert np.all(W[on & ~live] == 0)
+    act = net.forward(X[:256], 128, last_layer=0)
+    assert np.allclose(act.reshape(256, H, Mc).sum(2), 1.0, atol=1e-5) and act.min() >= 0
