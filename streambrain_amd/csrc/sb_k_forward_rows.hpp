@@ -19,6 +19,7 @@ struct ForwardRowsArgs {
   const int *rows;     // [H, cap], see k_mask_rows
   const int *row_cnt;  // [H]
   long cap;            // a multiple of 16
+  const T *xt;         // XT kernels: the batch in blocks of 16 rows (k_gather_rows_blocked), from row 0
 };
 
 // A workgroup owns 16 batch rows x one hypercolumn (as k_forward with FUSE).  The hypercolumn's row list
@@ -32,7 +33,9 @@ struct ForwardRowsArgs {
 // segment, which is padding where the list is shorter.
 // Requires M % VW == 0, Mc % VW == 0 and 16-byte aligned W.
 // RB: row blocks per workgroup, as in k_forward: 16*RB batch rows share every gathered W vector.
-template <typename T, int NG, int NWAVES, int RB = 1>
+// XT: x is read from the blocked copy `xt` instead of a.x: the 16 lanes p of an entry then read 16
+// consecutive elements (one 64-byte access) instead of one element each of 16 rows.
+template <typename T, int NG, int NWAVES, int RB = 1, bool XT = false>
 __global__ __launch_bounds__(64 * NWAVES)
 __attribute__((amdgpu_waves_per_eu(NWAVES >= 4 ? NWAVES / 4 : 1, NWAVES >= 4 ? NWAVES / 4 : 1)))
 void k_forward_rows(ForwardRowsArgs<T> ar) {
@@ -96,11 +99,16 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
   ForwardBias<T, NG, NWAVES>::load(bv, a.bias, j0, ncol);
 
   // x through a bounds-checked window over this tile's batch rows: rows past the batch and padding
-  // entries (offset kOutside) read zero
-  const BufferWindow<T> xwin(a.x + b0 * a.N, (a.B - b0) * a.N);
+  // entries (offset kOutside) read zero.  Blocked copy: block b0/16 + r starts N*16 elements after the
+  // previous one, lane p's row is element p of a column's run of 16.
+  const BufferWindow<T> xwin((XT ? ar.xt : a.x) + b0 * a.N,
+                             (XT ? (a.B + 15) / 16 * 16 - b0 : a.B - b0) * a.N);
   unsigned xat[RB];
 #pragma unroll
-  for (int r = 0; r < RB; r++) xat[r] = (unsigned)((long)(16 * r + p) * a.N * sizeof(T));
+  for (int r = 0; r < RB; r++)
+    xat[r] = XT ? (unsigned)(((long)r * a.N * 16 + p) * sizeof(T))
+                : (unsigned)((long)(16 * r + p) * a.N * sizeof(T));
+  constexpr unsigned XSTEP = (XT ? 16u : 1u) * (unsigned)sizeof(T);  // bytes between input columns
   // W: this lane's columns of group g, or the tile's first columns where the group hangs over the end
   // of the hypercolumn (those accumulator columns are never stored)
   const T *wcol[NG];
@@ -118,8 +126,7 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
 #pragma unroll
       for (int rb = 0; rb < RB; rb++) {
         T one[1];
-        xwin.template load_n<1>(one, r < 0 ? BufferWindow<T>::kOutside
-                                           : xat[rb] + (unsigned)r * (unsigned)sizeof(T));
+        xwin.template load_n<1>(one, r < 0 ? BufferWindow<T>::kOutside : xat[rb] + (unsigned)r * XSTEP);
         xo[rb][s] = one[0];
       }
       const long roff = (long)(r < 0 ? 0 : r) * a.M;

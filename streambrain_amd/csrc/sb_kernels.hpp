@@ -363,6 +363,37 @@ __global__ __launch_bounds__(256) void k_gather_rows(T *dst, const T *src, const
   for (long c = threadIdx.x; c < cols; c += 256) d[c] = s[c];
 }
 
+// The same rows in blocks of 16, column-major inside a block:  dst[(r / 16) * cols + c][r % 16] =
+// src[idx[r], c]  (idx == nullptr: src[r, c]); rows >= `rows` of the last block are written as zero.
+// In this layout the 16 batch rows of a forward tile lie side by side for every input column, so a
+// column picked by index costs one 64-byte access instead of 16 scattered ones.  One workgroup per block;
+// a thread reads 16 elements of one column (coalesced across threads) and writes them as one run.
+// plain (optional): the same rows in their plain layout, plain[r, :] = src[idx[r], :], from the same read.
+template <typename T>
+__global__ __launch_bounds__(256) void k_gather_rows_blocked(T *dst, T *plain, const T *src,
+                                                             const int64_t *idx, long rows, long cols) {
+  const long r0 = (long)blockIdx.x * 16;
+  const T *s[16];
+#pragma unroll
+  for (int k = 0; k < 16; k++) {
+    const long r = r0 + k;
+    s[k] = r < rows ? src + (idx ? idx[r] : r) * cols : nullptr;
+  }
+  T *d = dst + (long)blockIdx.x * cols * 16;
+  for (long c = threadIdx.x; c < cols; c += 256) {
+    T v[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) v[k] = s[k] ? s[k][c] : T(0);
+#pragma unroll
+    for (int k = 0; k < 16; k++) d[c * 16 + k] = v[k];
+    if (plain) {
+#pragma unroll
+      for (int k = 0; k < 16; k++)
+        if (s[k]) plain[(r0 + k) * cols + c] = v[k];
+    }
+  }
+}
+
 template <int UNUSED = 0>
 __global__ __launch_bounds__(256) void k_fill_bytes(uint8_t *dst, uint8_t value, size_t bytes) {
   const size_t stride = (size_t)gridDim.x * 256;

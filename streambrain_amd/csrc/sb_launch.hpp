@@ -70,11 +70,13 @@ int launch_forward_classify(hipStream_t st, T *act, const T *x, const T *W, cons
 // The same result for a layer whose W is zero wherever wmask is 0, from the per-hypercolumn lists of
 // connected rows that launch_mask_rows builds (rows: [H, cap] ascending indices, the rest -1; cap a
 // multiple of 16; row_cnt: [H]); forward_rows_supported says whether the kernel takes the shape.
+// x_blocked (optional): the same batch in blocks of 16 rows as launch_gather_rows_blocked lays them out,
+// starting at the batch's first row; then x itself is not read.
 template <typename T>
 bool forward_rows_supported(const T *W, long N, long H, long Mc);
 template <typename T>
 int launch_forward_rows(hipStream_t st, T *act, const T *x, const T *W, const T *bias, const int *rows,
-                        const int *row_cnt, long cap, long B, long N, long H, long Mc);
+                        const int *row_cnt, long cap, long B, long N, long H, long Mc, const T *x_blocked);
 // Lists of hypercolumns h0 .. h0 + count - 1 rebuilt from wmask.
 int launch_mask_rows(hipStream_t st, int *rows, int *row_cnt, const uint8_t *wmask, long N, long H,
                      long cap, long h0, long count);
@@ -113,6 +115,11 @@ int launch_argmax_rows(hipStream_t st, const T *act, const T *labels, long B, lo
                        unsigned long long *correct);
 template <typename T>
 int launch_gather_rows(hipStream_t st, T *dst, const T *src, const int64_t *idx, long rows, long cols);
+// dst[(r / 16) * cols + c][r % 16] = src[idx ? idx[r] : r, c], rows of the last block beyond `rows` zero:
+// ceil(rows / 16) * 16 * cols elements.  plain (optional) receives what launch_gather_rows would write.
+template <typename T>
+int launch_gather_rows_blocked(hipStream_t st, T *dst, T *plain, const T *src, const int64_t *idx, long rows,
+                               long cols);
 template <typename T>
 int launch_fill(hipStream_t st, T *dst, T value, size_t n);
 int launch_fill_bytes(hipStream_t st, void *dst, int value, size_t bytes);

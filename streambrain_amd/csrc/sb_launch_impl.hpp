@@ -153,27 +153,39 @@ static int forward_rows_variant(hipStream_t st, ForwardRowsArgs<T> a) {
   a.f.batch_tiles = cdiv(B, 16 * rb);
   const long grid = 8 * cdiv(a.f.col_tiles * a.f.batch_tiles, 8);
   SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
-  if constexpr (fits4) {
-    if (rb == 4) hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 4>), dim3((unsigned)grid), dim3(64 * NW), 0, st, a);
+  const dim3 g((unsigned)grid), blk(64 * NW);
+  if (a.xt) {  // the batch is also at hand in blocks of 16 rows
+    if constexpr (fits4) {
+      if (rb == 4) hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 4, true>), g, blk, 0, st, a);
+    }
+    if (rb == 4) {
+    } else if (rb == 2)
+      hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 2, true>), g, blk, 0, st, a);
+    else
+      hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 1, true>), g, blk, 0, st, a);
+  } else {
+    if constexpr (fits4) {
+      if (rb == 4) hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 4>), g, blk, 0, st, a);
+    }
+    if (rb == 4) {
+    } else if (rb == 2)
+      hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 2>), g, blk, 0, st, a);
+    else
+      hipLaunchKernelGGL((k_forward_rows<T, NG, NW>), g, blk, 0, st, a);
   }
-  if (rb == 4) {
-  } else if (rb == 2)
-    hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 2>), dim3((unsigned)grid), dim3(64 * NW), 0, st, a);
-  else
-    hipLaunchKernelGGL((k_forward_rows<T, NG, NW>), dim3((unsigned)grid), dim3(64 * NW), 0, st, a);
   SB_LAUNCH_CHECK();
   return 0;
 }
 
 template <typename T>
 int launch_forward_rows(hipStream_t st, T *act, const T *x, const T *W, const T *bias, const int *rows,
-                        const int *row_cnt, long cap, long B, long N, long H, long Mc) {
+                        const int *row_cnt, long cap, long B, long N, long H, long Mc, const T *x_blocked) {
   SB_REQUIRE(act && x && W && bias && rows && row_cnt, "null pointer");
   SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");
   SB_REQUIRE(H * Mc < (1L << 31) && N < (1L << 31), "dimension too large");
   SB_REQUIRE(cap > 0 && cap % 16 == 0, "row lists must be padded to a multiple of 16");
   SB_REQUIRE(forward_rows_supported<T>(W, N, H, Mc), "shape not supported by the row-list forward kernel");
-  ForwardRowsArgs<T> a{{act, x, W, bias, B, N, H * Mc, Mc, H, cdiv(B, 16)}, rows, row_cnt, cap};
+  ForwardRowsArgs<T> a{{act, x, W, bias, B, N, H * Mc, Mc, H, cdiv(B, 16)}, rows, row_cnt, cap, x_blocked};
   const long need = cdiv(Mc, 16 * Real<T>::VW);
   if (need <= 1) return forward_rows_variant<T, 1>(st, a);
   if (need <= 2) return forward_rows_variant<T, 2>(st, a);
@@ -380,6 +392,18 @@ int launch_gather_rows(hipStream_t st, T *dst, const T *src, const int64_t *idx,
 }
 
 template <typename T>
+int launch_gather_rows_blocked(hipStream_t st, T *dst, T *plain, const T *src, const int64_t *idx, long rows,
+                               long cols) {
+  SB_REQUIRE(dst && src, "null pointer");
+  SB_REQUIRE(rows > 0 && cols > 0 && cdiv(rows, 16) < (1L << 31), "bad shape");
+  ProfScope prof_(st, K_GATHER);
+  hipLaunchKernelGGL((k_gather_rows_blocked<T>), dim3((unsigned)cdiv(rows, 16)), dim3(256), 0, st, dst, plain,
+                     src, idx, rows, cols);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
 int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
   if (n == 0) return 0;
   SB_REQUIRE(dst, "null pointer");
@@ -398,7 +422,9 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
                                           unsigned long long *);                                      \
   template bool forward_rows_supported<T>(const T *, long, long, long);                               \
   template int launch_forward_rows<T>(hipStream_t, T *, const T *, const T *, const T *, const int *, \
-                                      const int *, long, long, long, long, long);                     \
+                                      const int *, long, long, long, long, long, const T *);          \
+  template int launch_gather_rows_blocked<T>(hipStream_t, T *, T *, const T *, const int64_t *, long, \
+                                             long);                                                  \
   template int launch_softmax<T>(hipStream_t, T *, long, long, long);                                 \
   template int launch_train_fused<T>(hipStream_t, const T *, const T *, T *, T *, const T *, const T *, \
                                      T *, T *, const uint8_t *, int, T *, T *, long, long, long, long, \

@@ -171,6 +171,8 @@ struct sb_net {
   std::vector<sb::Layer> layers;
   // training set in HBM, its per-epoch permuted copy and the permutation
   void *X = nullptr, *Y = nullptr, *Xp = nullptr, *Yp = nullptr;
+  long XpB_batch = 0;   // batch size XpB is valid for in the current epoch (0: not valid)
+  void *XpB = nullptr;  // Xp in blocks of 16 rows (k_gather_rows_blocked), for the first layer's forward over row lists
   long Ns = 0, NF = 0, NC = 0;
   int64_t *d_perm = nullptr;
   int64_t *h_perm = nullptr;  // pinned staging
@@ -180,6 +182,8 @@ struct sb_net {
 };
 
 namespace sb {
+
+static inline long cdiv_l(long a, long b) { return (a + b - 1) / b; }
 
 static int free_dev(void *&p) {
   if (p) SB_HIP(hipFree(p));
@@ -256,15 +260,16 @@ static int layer_check_masked(sb_net *net, Layer &L) {
   return 0;
 }
 
+// x_blocked: the same batch in blocks of 16 rows, or nullptr
 template <typename T>
-static int layer_forward(sb_net *net, Layer &L, const T *x, long B) {
+static int layer_forward(sb_net *net, Layer &L, const T *x, long B, const T *x_blocked = nullptr) {
   if (L.w_unchecked) {
     int rc = layer_check_masked<T>(net, L);
     if (rc) return rc;
   }
   if (L.rows && L.w_masked)
     return launch_forward_rows<T>(g_ctx.stream, (T *)L.act, x, (const T *)L.W, (const T *)L.bias, L.rows,
-                                  L.row_cnt, L.rows_cap, B, L.N, L.H, L.Mc);
+                                  L.row_cnt, L.rows_cap, B, L.N, L.H, L.Mc, x_blocked);
   return launch_forward<T>(g_ctx.stream, (T *)L.act, x, (const T *)L.W, (const T *)L.bias, B, L.N, L.H,
                            L.Mc, true);
 }
@@ -363,8 +368,20 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
   SB_HIP(hipMemcpyAsync(net->d_perm, net->h_perm, (size_t)Ns * sizeof(int64_t), hipMemcpyHostToDevice,
                         st));
   SB_HIP(hipEventRecord(net->perm_copied, st));
-  if ((rc = launch_gather_rows<T>(st, (T *)net->Xp, (const T *)net->X, net->d_perm, Ns, net->NF)))
-    return rc;
+  // A first layer that walks row lists reads its input column by column: it gets the shuffled images a
+  // second time, in blocks of 16 rows (batches must then start on block boundaries); one kernel writes
+  // both copies from one read.
+  if (net->layers[0].rows && maxB % 16 == 0) {
+    if (!net->XpB) SB_HIP(hipMalloc(&net->XpB, (size_t)cdiv_l(Ns, 16) * 16 * net->NF * net->esize));
+    if ((rc = launch_gather_rows_blocked<T>(st, (T *)net->XpB, (T *)net->Xp, (const T *)net->X, net->d_perm, Ns,
+                                            net->NF)))
+      return rc;
+    net->XpB_batch = maxB;
+  } else {
+    if ((rc = launch_gather_rows<T>(st, (T *)net->Xp, (const T *)net->X, net->d_perm, Ns, net->NF)))
+      return rc;
+    net->XpB_batch = 0;
+  }
   if (last)
     if ((rc = launch_gather_rows<T>(st, (T *)net->Yp, (const T *)net->Y, net->d_perm, Ns, net->NC)))
       return rc;
@@ -375,8 +392,9 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
     const long lo = i * maxB;
     const long B = (lo + maxB <= Ns) ? maxB : Ns - lo;
     const T *x = (const T *)net->Xp + lo * net->NF;
+    const T *xb = net->XpB_batch == maxB ? (const T *)net->XpB + lo * net->NF : nullptr;  // lo % 16 == 0
     for (int l = 0; l < layer; l++) {
-      if ((rc = layer_forward<T>(net, net->layers[l], x, B))) return rc;
+      if ((rc = layer_forward<T>(net, net->layers[l], x, B, l == 0 ? xb : nullptr))) return rc;
       x = (const T *)net->layers[l].act;
     }
     long h = -1;
@@ -393,7 +411,7 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
       // (_cpu_base_backend.py:290-295, 304-306); it has no effect on any state
       rc = layer_train_step<T>(target, x, (const T *)net->Yp + lo * net->NC, B, -1);
     } else {
-      if ((rc = layer_forward<T>(net, target, x, B))) return rc;
+      if ((rc = layer_forward<T>(net, target, x, B, layer == 0 ? xb : nullptr))) return rc;
       rc = layer_train_step<T>(target, x, (const T *)target.act, B, h);
     }
     if (rc) return rc;
@@ -425,9 +443,12 @@ static int net_forward_batches(sb_net *net, const void *h_images, const void *h_
   chunk = chunk / maxB * maxB;
   if (chunk < maxB) chunk = maxB;
   if (chunk > n) chunk = n;
-  void *dX = nullptr, *dY = nullptr;
+  void *dX = nullptr, *dY = nullptr, *dXB = nullptr;
   int32_t *dP = nullptr;
   SB_HIP(hipMalloc(&dX, (size_t)chunk * NF * sizeof(T)));
+  // a first layer that walks row lists also gets every chunk in blocks of 16 rows (see net_train_batches)
+  const bool blocked = net->layers[0].rows && maxB % 16 == 0;
+  if (blocked) SB_HIP(hipMalloc(&dXB, (size_t)cdiv_l(chunk, 16) * 16 * NF * sizeof(T)));
   if (h_labels) SB_HIP(hipMalloc(&dY, (size_t)chunk * NC * sizeof(T)));
   if (h_pred) SB_HIP(hipMalloc((void **)&dP, (size_t)chunk * sizeof(int32_t)));
   if (h_labels) {
@@ -441,9 +462,11 @@ static int net_forward_batches(sb_net *net, const void *h_images, const void *h_
     if (h_labels)
       SB_HIP(hipMemcpy(dY, (const T *)h_labels + c0 * NC, (size_t)rows * NC * sizeof(T),
                        hipMemcpyHostToDevice));
+    if (blocked) rc = launch_gather_rows_blocked<T>(st, (T *)dXB, (T *)nullptr, (const T *)dX, nullptr, rows, NF);
     for (long lo = 0; lo < rows && !rc; lo += maxB) {
       const long B = (lo + maxB <= rows) ? maxB : rows - lo;
       const T *x = (const T *)dX + lo * NF;
+      const T *xb = blocked ? (const T *)dXB + lo * NF : nullptr;
       const bool classify = h_labels || h_pred;
       for (int l = 0; l <= last_layer && !rc; l++) {
         Layer &L = net->layers[l];
@@ -453,7 +476,7 @@ static int net_forward_batches(sb_net *net, const void *h_images, const void *h_
                                           L.Mc, true, h_labels ? (const T *)dY + lo * NC : nullptr,
                                           dP ? dP + lo : nullptr, net->d_correct);
         else
-          rc = layer_forward<T>(net, L, x, B);
+          rc = layer_forward<T>(net, L, x, B, l == 0 ? xb : nullptr);
         x = (const T *)L.act;
       }
       if (rc) break;
@@ -475,6 +498,7 @@ static int net_forward_batches(sb_net *net, const void *h_images, const void *h_
     *correct = (int64_t)cnt;
   }
   SB_HIP(hipFree(dX));
+  if (dXB) SB_HIP(hipFree(dXB));
   if (dY) SB_HIP(hipFree(dY));
   if (dP) SB_HIP(hipFree(dP));
   return rc;
@@ -622,7 +646,8 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
   int sb_compute_activation_rows_##SFX(T *act, const T *x, const T *W, const T *bias, const int *rows, \
                                        const int *row_cnt, long cap, long B, long N, long H, long Mc) { \
     SB_READY();                                                                                        \
-    return launch_forward_rows<T>(g_ctx.stream, act, x, W, bias, rows, row_cnt, cap, B, N, H, Mc);     \
+    return launch_forward_rows<T>(g_ctx.stream, act, x, W, bias, rows, row_cnt, cap, B, N, H, Mc,      \
+                                  nullptr);                                                            \
   }                                                                                                    \
   int sb_update_weights_##SFX(T *Ci, T *Cj, T *Cij, const T *a_i, const T *a_o, T taupdt, T *W,        \
                               T cthr, long B, long N, long M) {                                        \
@@ -707,6 +732,8 @@ int sb_net_training_done(sb_net *net) {
   int rc = 0;
   void *p = net->d_perm;
   rc |= free_dev(net->X); rc |= free_dev(net->Y); rc |= free_dev(net->Xp); rc |= free_dev(net->Yp);
+  rc |= free_dev(net->XpB);
+  net->XpB_batch = 0;
   rc |= free_dev(p);
   net->d_perm = nullptr;
   if (net->h_perm) SB_HIP(hipHostFree(net->h_perm));
