@@ -89,10 +89,16 @@ int sb_compute_activation_f64(double *d_act, const double *d_x, const double *d_
 int sb_mask_rows(int *d_rows, int *d_row_cnt, const unsigned char *d_wmask, long N, long H, long cap);
 int sb_compute_activation_rows_f32(float *d_act, const float *d_x, const float *d_W,
                                    const float *d_bias, const int *d_rows, const int *d_row_cnt,
-                                   long cap, long B, long N, long H, long Mc);
+                                   long cap, long B, long N, long H, long Mc, const float *d_x_blocked);
 int sb_compute_activation_rows_f64(double *d_act, const double *d_x, const double *d_W,
                                    const double *d_bias, const int *d_rows, const int *d_row_cnt,
-                                   long cap, long B, long N, long H, long Mc);
+                                   long cap, long B, long N, long H, long Mc, const double *d_x_blocked);
+/* d_x_blocked (optional, may be NULL): the same batch in blocks of 16 rows, as sb_rows_in_blocks lays it
+ * out: d_dst[(r / 16) * cols + c][r % 16] = d_src[r, c], ceil(rows / 16) * 16 * cols elements, rows past
+ * the last one zero.  The kernel then reads a picked input column of 16 batch rows as one 64-byte run
+ * instead of 16 scattered elements, and d_x itself is not read. */
+int sb_rows_in_blocks_f32(float *d_dst, const float *d_src, long rows, long cols);
+int sb_rows_in_blocks_f64(double *d_dst, const double *d_src, long rows, long cols);
 
 /* Ci, Cj, Cij moving averages (clamped at 0) and W = log(max(Cij,cthr^4)/(Ci*Cj)) with rows
  * Ci<cthr and columns Cj<cthr zeroed; all in place; W is the unmasked weight.

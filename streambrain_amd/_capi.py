@@ -22,7 +22,8 @@ _KERNEL_SIGS = {
     "sb_update_state": lambda R: [_P, _P, _P, _P, _L, _L, _L],
     "sb_softmax_minicolumns": lambda R: [_P, _L, _L, _L],
     "sb_compute_activation": lambda R: [_P, _P, _P, _P, _L, _L, _L, _L],
-    "sb_compute_activation_rows": lambda R: [_P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _L],
+    "sb_compute_activation_rows": lambda R: [_P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _P],
+    "sb_rows_in_blocks": lambda R: [_P, _P, _L, _L],
     "sb_update_weights": lambda R: [_P, _P, _P, _P, _P, R, _P, R, _L, _L, _L],
     "sb_update_bias": lambda R: [_P, _P, R, _L],
     "sb_update_bias_regularized": lambda R: [_P, _P, _P, R, R, R, R, _L],

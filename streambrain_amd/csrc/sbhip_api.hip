@@ -644,10 +644,15 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
     return launch_forward<T>(g_ctx.stream, act, x, W, bias, B, N, H, Mc, true);                        \
   }                                                                                                    \
   int sb_compute_activation_rows_##SFX(T *act, const T *x, const T *W, const T *bias, const int *rows, \
-                                       const int *row_cnt, long cap, long B, long N, long H, long Mc) { \
+                                       const int *row_cnt, long cap, long B, long N, long H, long Mc,  \
+                                       const T *x_blocked) {                                           \
     SB_READY();                                                                                        \
     return launch_forward_rows<T>(g_ctx.stream, act, x, W, bias, rows, row_cnt, cap, B, N, H, Mc,      \
-                                  nullptr);                                                            \
+                                  x_blocked);                                                          \
+  }                                                                                                    \
+  int sb_rows_in_blocks_##SFX(T *dst, const T *src, long rows, long cols) {                            \
+    SB_READY();                                                                                        \
+    return launch_gather_rows_blocked<T>(g_ctx.stream, dst, (T *)nullptr, src, nullptr, rows, cols);   \
   }                                                                                                    \
   int sb_update_weights_##SFX(T *Ci, T *Cj, T *Cij, const T *a_i, const T *a_o, T taupdt, T *W,        \
                               T cthr, long B, long N, long M) {                                        \

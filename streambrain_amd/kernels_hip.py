@@ -73,8 +73,18 @@ def mask_rows(wmask):
     return d_rows.numpy(), d_cnt.numpy()
 
 
-def compute_activation_rows(weights, bias, inputs, wmask, hypercolumns, minicolumns):
-    """compute_activation for weights that are zero wherever wmask is 0, over the connected rows only."""
+def rows_in_blocks(a):
+    """a[rows, cols] in blocks of 16 rows, column-major inside a block; rows past the last one zero."""
+    a = np.ascontiguousarray(a)
+    rows, cols = a.shape
+    d = DeviceArray(((rows + 15) // 16 * 16 * cols,), a.dtype)
+    check(_fn("sb_rows_in_blocks", a.dtype)(d.ptr, _dev(a).ptr, rows, cols))
+    return d
+
+
+def compute_activation_rows(weights, bias, inputs, wmask, hypercolumns, minicolumns, blocked=False):
+    """compute_activation for weights that are zero wherever wmask is 0, over the connected rows only;
+    blocked: the kernel reads the inputs from their copy in blocks of 16 rows."""
     dt = weights.dtype
     f = _fn("sb_compute_activation_rows", dt)
     B, N = inputs.shape
@@ -84,8 +94,9 @@ def compute_activation_rows(weights, bias, inputs, wmask, hypercolumns, minicolu
     d_act = DeviceArray((B, M), dt)
     d_x, d_w, d_b = _dev(inputs, dt), _dev(weights, dt), _dev(bias, dt)
     d_rows, d_cnt = _dev(rows), _dev(cnt)
+    d_xb = rows_in_blocks(np.asarray(inputs, dtype=dt)) if blocked else None
     check(f(d_act.ptr, d_x.ptr, d_w.ptr, d_b.ptr, d_rows.ptr, d_cnt.ptr, rows.shape[1], B, N,
-            hypercolumns, minicolumns))
+            hypercolumns, minicolumns, d_xb.ptr if blocked else None))
     return d_act.numpy()
 
 

@@ -51,6 +51,20 @@ def test_update_state(k, oracle, dtype, B, N, M):
 
 
 # ------------------------------------------------------------- forward over the connected rows only
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("rows,cols", [(1, 1), (16, 5), (37, 300), (128, 1568)])
+def test_rows_in_blocks(k, dtype, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    a = rng.random((rows, cols)).astype(dtype)
+    got = k.rows_in_blocks(a).numpy()
+    nb = (rows + 15) // 16
+    want = np.zeros((nb * 16, cols), dtype=dtype)
+    want[:rows] = a
+    want = want.reshape(nb, 16, cols).transpose(0, 2, 1).reshape(-1)
+    assert np.array_equal(got, want)
+
+
+
 @pytest.mark.parametrize("N,H,density", [(1, 1, 1.0), (40, 3, 0.3), (1568, 30, 0.1), (300, 5, 0.0),
                                          (257, 4, 0.05), (64, 2, 1.0)])
 def test_mask_rows(k, N, H, density):
@@ -75,7 +89,8 @@ def test_mask_rows(k, N, H, density):
                                               # many tiles: 32 and 64 batch rows per workgroup, ragged
                                               (1000, 300, 32, 100, 0.2), (2030, 200, 64, 100, 0.3),
                                               (12, 40, 2, 224, 0.5)])
-def test_compute_activation_rows(k, oracle, dtype, B, N, H, Mc, density):
+@pytest.mark.parametrize("blocked", [False, True])
+def test_compute_activation_rows(k, oracle, dtype, B, N, H, Mc, density, blocked):
     """The row-list forward kernel against the dense reference computation on the masked weights."""
     if dtype == np.float32 and Mc % 4:
         pytest.skip("float32 needs minicolumns divisible by 4")
@@ -87,7 +102,7 @@ def test_compute_activation_rows(k, oracle, dtype, B, N, H, Mc, density):
     x = rng.random((B, N)).astype(dtype)
     W = (0.1 * rng.standard_normal((N, M))).astype(dtype) * np.repeat(wmask, Mc, axis=1).astype(dtype)
     b = (0.1 * rng.random(M)).astype(dtype)
-    got = k.compute_activation_rows(W, b, x, wmask, H, Mc)
+    got = k.compute_activation_rows(W, b, x, wmask, H, Mc, blocked=blocked)
     ref = oracle.update_state(np.zeros((B, M), dtype=dtype), W, b, x)
     ref = oracle.softmax_minicolumns(ref, H, Mc)
     scale = max(1.0, np.sqrt(N / 64.0)) if dtype == np.float32 else 4.0

@@ -122,8 +122,15 @@ def _check_layer_at_size(dtype, B, N, H, Mc, density, seed):
         _capi.check(lib.sb_mask_rows(d_rows.ptr, d_cnt.ptr, d_m.ptr, N, H, cap))
         d_act2 = DeviceArray((B, M), dtype)
         _capi.check(fn("sb_compute_activation_rows")(d_act2.ptr, d_xs.ptr, d_w.ptr, d_bias.ptr, d_rows.ptr,
-                                                     d_cnt.ptr, cap, B, N, H, Mc))
+                                                     d_cnt.ptr, cap, B, N, H, Mc, None))
         assert np.array_equal(d_cnt.numpy(), np.count_nonzero(wmask, axis=0))
+        assert np.max(np.abs(d_act2.numpy() - act)) <= 16 * tol
+        # ... and the same from the inputs laid out in blocks of 16 rows
+        d_xb = DeviceArray(((B + 15) // 16 * 16 * N,), dtype)
+        _capi.check(fn("sb_rows_in_blocks")(d_xb.ptr, d_xs.ptr, B, N))
+        _capi.check(lib.sb_fill_bytes(d_act2.ptr, 0, B * M * es))
+        _capi.check(fn("sb_compute_activation_rows")(d_act2.ptr, d_xs.ptr, d_w.ptr, d_bias.ptr, d_rows.ptr,
+                                                     d_cnt.ptr, cap, B, N, H, Mc, d_xb.ptr))
         assert np.max(np.abs(d_act2.numpy() - act)) <= 16 * tol
 
 
