@@ -79,10 +79,12 @@ def _mask_diff(a, b):
     return int((a != b).sum())
 
 
-def test_small_network_epochs_with_rewiring_f64(hb):
-    # 3 + 2 epochs, 13 batches with a short last one, rewiring from the second epoch on: in float64
-    # the whole trajectory, masks included, is reproduced.
-    (g, r), (Xt, Yt) = _run_both(hb, np.float64, n_pix=60, H=4, Mc=10, n_out=5, Ns=200, Nt=50, B=16,
+@pytest.mark.parametrize("B", [16, 20])
+def test_small_network_epochs_with_rewiring_f64(hb, B):
+    # 3 + 2 epochs, 13 (10) batches with a short last one, rewiring from the second epoch on: in float64
+    # the whole trajectory, masks included, is reproduced.  (Batches of 16 let the first layer's forward
+    # read its input in blocks of 16 rows, batches of 20 do not.)
+    (g, r), (Xt, Yt) = _run_both(hb, np.float64, n_pix=60, H=4, Mc=10, n_out=5, Ns=200, Nt=50, B=B,
                                  e1=3, e2=2, hp=dict(MNIST_HP, l1_density=0.3), data_seed=11)
     assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
     _compare_states(g, r, 1e-10)
