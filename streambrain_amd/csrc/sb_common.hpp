@@ -215,6 +215,26 @@ __device__ __forceinline__ T row16_reduce(T v, Op op) {
   return v;
 }
 
+// Division of n < 2^31 by a divisor fixed per launch, as a multiplication: the host prepares
+// m = ceil(2^k / d) with k = 31 + ceil(log2 d), and  n / d == (n * m) >> k  for every n < 2^31
+// (m * d - 2^k < 2^(k-31)).  Three instructions instead of the two dozen of a 32-bit division, and on
+// the scalar unit when n is uniform.
+struct FastDiv {
+  uint32_t m, k;
+  static FastDiv of(long d) {
+    uint32_t s = 0;
+    while ((1L << s) < d) s++;
+    FastDiv f;
+    f.k = 31 + s;
+    const unsigned __int128 p = (unsigned __int128)1 << f.k;
+    f.m = (uint32_t)(p / (unsigned long)d + (p % (unsigned long)d ? 1 : 0));
+    return f;
+  }
+  __host__ __device__ __forceinline__ uint32_t div(uint32_t n) const {
+    return (uint32_t)(((uint64_t)n * m) >> k);
+  }
+};
+
 // The weight of one synapse from its traces, shared by the trace/weight kernel and the rewiring
 // kernels so both see bit-identical values:  log(max(cij, cthr^4) / (ci * cj)) evaluated as
 // log(max(cij, cthr^4) * (1/ci) * (1/cj)).  rci / rcj are the reciprocals, or a negative number when

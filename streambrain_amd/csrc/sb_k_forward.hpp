@@ -33,6 +33,7 @@ struct ForwardArgs {
   const T *bias;
   long B, N, M, Mc;
   long col_tiles, batch_tiles;
+  FastDiv by_batch_tiles;  // division by batch_tiles (set by the launcher along with it)
 };
 
 // Column layout of a tile, shared by the kernels below: NG groups of 16 lanes-columns, group g holding
@@ -212,7 +213,7 @@ void k_forward(ForwardArgs<T> a) {
   const long per_xcd = (ntiles + 7) / 8;
   const long tile = (long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (tile >= ntiles) return;  // whole workgroup, before any barrier
-  const long ct = tile / a.batch_tiles, bt = tile % a.batch_tiles;
+  const long ct = a.by_batch_tiles.div((uint32_t)tile), bt = tile - ct * a.batch_tiles;  // tile < 2^31
 
   const int tid = threadIdx.x, lane = tid & 63, p = lane & 15, q = lane >> 4;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, in a scalar register: uniform branches

@@ -57,7 +57,7 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
   const long per_xcd = (ntiles + 7) / 8;
   const long tile = (long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (tile >= ntiles) return;  // whole workgroup, before any barrier
-  const long ct = tile / a.batch_tiles, bt = tile % a.batch_tiles;
+  const long ct = a.by_batch_tiles.div((uint32_t)tile), bt = tile - ct * a.batch_tiles;  // tile < 2^31
 
   const int tid = threadIdx.x, lane = tid & 63, p = lane & 15, q = lane >> 4;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -61,6 +61,7 @@ struct TrainArgs {
   T tau, omt, fB, invB, cthr, cthr4;
   T khalf, pmin, taubdt;
   long tiles_i, tiles_j;
+  FastDiv by_tiles_i, by_Mc;  // divisions by tiles_i and by Mc
 };
 
 // MB: mask bytes fetched per vector of VW columns -- 1 when Mc is a multiple of VW (every vector lies
@@ -94,7 +95,7 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   const unsigned per_xcd = (ntiles + 7) / 8;
   const unsigned tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (tile >= ntiles) return;  // whole workgroup, before any barrier
-  const long jt = tile / (unsigned)a.tiles_i, it = tile % (unsigned)a.tiles_i;
+  const long jt = a.by_tiles_i.div(tile), it = tile - (unsigned)jt * (unsigned)a.tiles_i;
   const long i0 = it * TS, j0 = jt * TS;
 
   // thread's share of the tile in row-major order: VW columns of PASSES rows
@@ -151,7 +152,7 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   if (a.wmask) {
     uint32_t hc[MB];
 #pragma unroll
-    for (int e = 0; e < MB; e++) hc[e] = ecol + e < a.M ? (uint32_t)(ecol + e) / (uint32_t)a.Mc : 0u;
+    for (int e = 0; e < MB; e++) hc[e] = ecol + e < a.M ? a.by_Mc.div((uint32_t)(ecol + e)) : 0u;
 #pragma unroll
     for (int k = 0; k < PASSES; k++) {
       const long row = i0 + er + RPP * k;

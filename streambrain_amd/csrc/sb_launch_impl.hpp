@@ -20,6 +20,7 @@ static inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 template <typename T, int NG, bool FUSE>
 static int forward_variant(hipStream_t st, ForwardArgs<T> a, bool vec) {
   ProfScope prof_(st, K_FORWARD);
+  a.by_batch_tiles = FastDiv::of(a.batch_tiles);
   // 8 workgroup ids per round of XCDs; ids beyond the last tile exit at once
   const long ntiles = a.col_tiles * a.batch_tiles;
   const long grid = 8 * cdiv(ntiles, 8);
@@ -101,6 +102,7 @@ int launch_forward_classify(hipStream_t st, T *act, const T *x, const T *W, cons
         // (32-bit byte offsets inside the tile's rows)
         while (rb > 1 && 16 * rb * N * (long)sizeof(T) >= (1L << 31)) rb /= 2;
         a.batch_tiles = cdiv(B, 16 * rb);
+        a.by_batch_tiles = FastDiv::of(a.batch_tiles);
         ProfScope prof_(st, K_FORWARD);
         const long grid = 8 * cdiv(a.col_tiles * a.batch_tiles, 8);
         SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
@@ -151,6 +153,7 @@ static int forward_rows_variant(hipStream_t st, ForwardRowsArgs<T> a) {
   // (32-bit byte offsets inside the tile's rows)
   while (rb > 1 && 16 * rb * a.f.N * (long)sizeof(T) >= (1L << 31)) rb /= 2;
   a.f.batch_tiles = cdiv(B, 16 * rb);
+  a.f.by_batch_tiles = FastDiv::of(a.f.batch_tiles);
   const long grid = 8 * cdiv(a.f.col_tiles * a.f.batch_tiles, 8);
   SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
   const dim3 g((unsigned)grid), blk(64 * NW);
@@ -229,6 +232,7 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   a.tau = s.tau; a.omt = s.omt; a.fB = (T)B; a.invB = (T)1 / (T)B; a.cthr = s.cthr; a.cthr4 = s.cthr4;
   a.khalf = khalf; a.pmin = pmin; a.taubdt = taubdt;
   a.tiles_i = cdiv(N, 64); a.tiles_j = cdiv(M, 64);
+  a.by_tiles_i = FastDiv::of(a.tiles_i); a.by_Mc = FastDiv::of(Mc);
   if (M <= 32) {  // a handful of output units: plain vector arithmetic
     const long rows = 256 / M;
     SB_REQUIRE(cdiv(N, rows) < (1L << 31), "too many rows for one launch");
