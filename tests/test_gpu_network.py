@@ -339,3 +339,58 @@ def test_full_size_epochs_keep_the_invariants_f32(hb):
     assert np.all(W[on & ~live] == 0)
     act = net.forward(X[:256], 128, last_layer=0)
     assert np.allclose(act.reshape(256, H, Mc).sum(2), 1.0, atol=1e-5) and act.min() >= 0
+
+
+def test_example_script_flow_through_the_package(tmp_path, monkeypatch):
+    """The flow of the reference's example script (train.py:9-23, 144-202 there) on idx-ubyte files
+    written here: read the files, complementary coding, `import BCPNN` with BCPNN_BACKEND=hip, the two
+    layers with the script's positional arguments, fit layer by layer, evaluate on both sets.  A learnable
+    toy problem (the class is which block of pixels is lit), so the accuracy says the pieces fit together."""
+    import importlib
+    import sys
+    from streambrain_amd import datasets
+
+    rng = np.random.default_rng(3)
+
+    def make(n):
+        lab = rng.integers(0, 10, n).astype(np.uint8)
+        px = (rng.random((n, 784)) < 0.03) * rng.integers(1, 120, (n, 784))
+        for k in range(n):
+            c = int(lab[k])
+            px[k, 78 * c:78 * c + 78] = rng.integers(150, 256, 78)
+        return px.astype(np.uint8), lab
+
+    def write(name, header, payload):
+        with open(tmp_path / name, "wb") as f:
+            f.write(bytes(header))
+            f.write(payload.tobytes())
+
+    for split, n in (("train", 1280), ("t10k", 320)):
+        px, lab = make(n)
+        write(f"{split}-images", [0, 0, 8, 3] + [0] * 12, px)
+        write(f"{split}-labels", [0, 0, 8, 1] + [0] * 4, lab)
+
+    monkeypatch.setenv("BCPNN_BACKEND", "hip")
+    sys.modules.pop("BCPNN", None)
+    BCPNN = importlib.import_module("BCPNN")
+    assert BCPNN.backend() == "hip"
+
+    precision = np.float32
+    np.random.seed(0)
+    train_x, train_y = datasets.load_mnist(tmp_path / "train-images", tmp_path / "train-labels", precision)
+    test_x, test_y = datasets.load_mnist(tmp_path / "t10k-images", tmp_path / "t10k-labels", precision)
+    train_x, test_x = datasets.complementary(train_x), datasets.complementary(test_x)
+    batch = 128
+    hp = MNIST_HP
+    net = BCPNN.Network(precision)
+    net.add_layer(BCPNN.StructuralPlasticityLayer(784 * 2, 15, 20, hp["l1_taupdt"] * 4, hp["l1_khalf"],
+                                                  hp["l1_pmin"], hp["l1_taubdt"], 0.3, 16, (1, 1 / 20, 1 / 20)))
+    net.add_layer(BCPNN.DenseLayer(15 * 20, 1, 10, hp["l2_taupdt"] * 40, (1 / 20, 1 / 10, 1 / 200)))
+    net.fit(train_x, train_y, batch, [(0, 4), (1, 4)])
+    correct, total = net.evaluate(train_x, train_y, batch)
+    assert total == 1280 and 0 <= correct <= total
+    train_acc = correct / total
+    correct, total = net.evaluate(test_x, test_y, batch)
+    assert total == 320
+    test_acc = correct / total
+    assert train_acc > 0.5 and test_acc > 0.5, (train_acc, test_acc)
