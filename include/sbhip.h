@@ -100,6 +100,22 @@ int sb_compute_activation_rows_f64(double *d_act, const double *d_x, const doubl
 int sb_rows_in_blocks_f32(float *d_dst, const float *d_src, long rows, long cols);
 int sb_rows_in_blocks_f64(double *d_dst, const double *d_src, long rows, long cols);
 
+/* The two halves of update_weights as the reference's cuda kernel set has them
+ * (BCPNN/backend/_kernels/kernels_cuda.py:40-59), and its separate bias step (:18-26):
+ *   sb_update_counters        Ci, Cj, Cij moving averages only (kernels_openmp_internal.cc:89-190)
+ *   sb_weights_from_counters  W from the traces as they are (:192-199), unmasked
+ *   sb_add_bias               act[b, j] += bias[j] */
+int sb_update_counters_f32(float *d_Ci, float *d_Cj, float *d_Cij, const float *d_a_i, const float *d_a_o,
+                           float taupdt, long B, long N, long M);
+int sb_update_counters_f64(double *d_Ci, double *d_Cj, double *d_Cij, const double *d_a_i,
+                           const double *d_a_o, double taupdt, long B, long N, long M);
+int sb_weights_from_counters_f32(float *d_W, const float *d_Ci, const float *d_Cj, const float *d_Cij,
+                                 float cthr, long N, long M);
+int sb_weights_from_counters_f64(double *d_W, const double *d_Ci, const double *d_Cj, const double *d_Cij,
+                                 double cthr, long N, long M);
+int sb_add_bias_f32(float *d_act, const float *d_bias, long B, long M);
+int sb_add_bias_f64(double *d_act, const double *d_bias, long B, long M);
+
 /* Ci, Cj, Cij moving averages (clamped at 0) and W = log(max(Cij,cthr^4)/(Ci*Cj)) with rows
  * Ci<cthr and columns Cj<cthr zeroed; all in place; W is the unmasked weight.
  * replaces update_weights_float32/64 -> vectorized_updateWeights,

@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256) void k_train_skinny(TrainArgs<T> a) {
   const T wgt = weight_from_traces<T>(cn, trace_reciprocal<T>(ci, a.cthr), trace_reciprocal<T>(cj, a.cthr),
                                       a.cthr4);
   const bool on = a.wmask == nullptr || a.wmask[i * a.H + j / (int)a.Mc] != 0;
-  a.W[i * a.M + j] = on ? wgt : T(0);
+  if (a.W) a.W[i * a.M + j] = on ? wgt : T(0);
 }
 
 }  // namespace sb

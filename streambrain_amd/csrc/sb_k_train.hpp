@@ -48,7 +48,7 @@ struct TrainArgs {
   const T *x;  // [B,N]
   const T *y;  // [B,M]
   T *Cij;
-  T *W;
+  T *W;          // nullptr: the traces are updated and no weights are written
   const T *Ci;   // old traces (read)
   const T *Cj;
   T *Ci_next;    // new traces (written by the first tile column / row)
@@ -303,6 +303,7 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
     bool connected = !masked;
 #pragma unroll
     for (int e = 0; e < MB; e++) connected = connected || mb[k][e] != 0;
+    if (a.W == nullptr) continue;
     if (a.w_masked && __builtin_amdgcn_ballot_w64(connected) == 0) continue;
     T wv[VW];
 #pragma unroll

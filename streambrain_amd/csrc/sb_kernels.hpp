@@ -66,6 +66,26 @@ __global__ __launch_bounds__(256) void k_update_bias_regularized(T *bias, T *kbi
   kbi[j] = kb;
 }
 
+// act[b, j] += bias[j]   (the separate bias step of the reference's cuda kernel set, kernels_cuda.py:18-26)
+template <typename T>
+__global__ __launch_bounds__(256) void k_add_bias(T *act, const T *bias, long B, long M) {
+  const long total = B * M;
+  const long stride = (long)gridDim.x * 256;
+  for (long e = (long)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) act[e] += bias[e % M];
+}
+
+// W[i, j] from the traces as they are (omp.cc:192-199 on its own; kernels_cuda.py:51-59 has it as a
+// separate step): the same expression as the fused training kernel.
+template <typename T>
+__global__ __launch_bounds__(256) void k_weights_from_traces(T *W, const T *Ci, const T *Cj, const T *Cij,
+                                                             T cthr, T cthr4, long N, long M) {
+  for (long i = blockIdx.x; i < N; i += gridDim.x) {
+    const T rci = trace_reciprocal<T>(Ci[i], cthr);
+    for (long j = threadIdx.x; j < M; j += 256)
+      W[i * M + j] = weight_from_traces<T>(Cij[i * M + j], rci, trace_reciprocal<T>(Cj[j], cthr), cthr4);
+  }
+}
+
 // omp.cc:322-335
 template <typename T>
 __global__ __launch_bounds__(256) void k_apply_mask(T *W, const uint8_t *wmask, long N, long M, long H,

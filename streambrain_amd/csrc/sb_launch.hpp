@@ -84,12 +84,19 @@ template <typename T>
 int launch_softmax(hipStream_t st, T *act, long B, long H, long Mc);
 // Fused Ci/Cj/Cij + weights (+ regularised bias when bias_mode == 1, + mask when wmask != nullptr).
 // Reads the old traces from Ci/Cj and writes the new ones to Ci_next/Cj_next (distinct buffers).
+// W == nullptr: the traces only.
 // w_masked: the caller vouches that W is zero wherever wmask is 0; such entries may then be left alone.
 template <typename T>
 int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci, const T *Cj,
                        T *Ci_next, T *Cj_next, const uint8_t *wmask, int bias_mode, T *bias, T *kbi,
                        long B, long N, long H, long Mc, T taupdt, T cthr, T khalf, T pmin, T taubdt,
                        bool w_masked);
+// W from the traces as they are, the fused kernel's expression (unmasked).
+template <typename T>
+int launch_weights_from_traces(hipStream_t st, T *W, const T *Ci, const T *Cj, const T *Cij, T cthr, long N,
+                               long M);
+template <typename T>
+int launch_add_bias(hipStream_t st, T *act, const T *bias, long B, long M);
 template <typename T>
 int launch_update_bias(hipStream_t st, T *bias, const T *Cj, T cthr, long M);
 template <typename T>

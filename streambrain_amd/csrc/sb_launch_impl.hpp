@@ -217,7 +217,7 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
                        long B, long N, long H, long Mc, T taupdt, T cthr, T khalf, T pmin, T taubdt,
                        bool w_masked) {
   constexpr int VW = Real<T>::VW;
-  SB_REQUIRE(x && y && Cij && W && Ci && Cj && Ci_next && Cj_next, "null pointer");
+  SB_REQUIRE(x && y && Cij && Ci && Cj && Ci_next && Cj_next, "null pointer");  // W may be null: traces only
   SB_REQUIRE(Ci != Ci_next && Cj != Cj_next, "old and new traces must be distinct buffers");
   SB_REQUIRE(bias_mode == 0 || (bias && kbi), "bias update needs bias and kbi");
   SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");
@@ -247,7 +247,7 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   SB_REQUIRE(64 * (N > M ? N : M) * (long)sizeof(T) <= (1L << 31),
              "layer too wide: 64 rows of it must stay below 2 GiB");
   const bool vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(y) && aligned16(Cij) &&
-                   aligned16(W);
+                   aligned16(W);  // (a null W counts as aligned)
   // 8 workgroup ids per round of XCDs; ids beyond the last tile exit at once
   const dim3 grid((unsigned)(8 * cdiv(a.tiles_i * a.tiles_j, 8)));
   // batch rows staged per chunk: 16 KiB of LDS per workgroup, so five workgroups share a CU
@@ -262,6 +262,30 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
     hipLaunchKernelGGL((k_train_fused<T, KCH, false, 1>), grid, dim3(256), 0, st, a);
   else
     hipLaunchKernelGGL((k_train_fused<T, KCH, false, VW>), grid, dim3(256), 0, st, a);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
+int launch_weights_from_traces(hipStream_t st, T *W, const T *Ci, const T *Cj, const T *Cij, T cthr, long N,
+                               long M) {
+  SB_REQUIRE(W && Ci && Cj && Cij, "null pointer");
+  SB_REQUIRE(N > 0 && M > 0, "sizes must be positive");
+  const TraceScalars<T> s = TraceScalars<T>::from(T(0), cthr);
+  ProfScope prof_(st, K_APPLY_MASK);
+  hipLaunchKernelGGL((k_weights_from_traces<T>), dim3((unsigned)(N < 8192 ? N : 8192)), dim3(256), 0, st, W, Ci,
+                     Cj, Cij, cthr, s.cthr4, N, M);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
+int launch_add_bias(hipStream_t st, T *act, const T *bias, long B, long M) {
+  SB_REQUIRE(act && bias, "null pointer");
+  SB_REQUIRE(B > 0 && M > 0, "sizes must be positive");
+  const long blocks = cdiv(B * M, 256) < 8192 ? cdiv(B * M, 256) : 8192;
+  ProfScope prof_(st, K_UPDATE_BIAS);
+  hipLaunchKernelGGL((k_add_bias<T>), dim3((unsigned)blocks), dim3(256), 0, st, act, bias, B, M);
   SB_LAUNCH_CHECK();
   return 0;
 }
@@ -434,6 +458,9 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
                                      T *, T *, const uint8_t *, int, T *, T *, long, long, long, long, \
                                      T, T, T, T, T, bool);                                             \
   template int launch_update_bias<T>(hipStream_t, T *, const T *, T, long);                           \
+  template int launch_weights_from_traces<T>(hipStream_t, T *, const T *, const T *, const T *, T,    \
+                                             long, long);                                             \
+  template int launch_add_bias<T>(hipStream_t, T *, const T *, long, long);                           \
   template int launch_update_bias_regularized<T>(hipStream_t, T *, T *, const T *, T, T, T, T, long); \
   template int launch_update_mask<T>(hipStream_t, uint8_t *, const T *, const T *, const T *,         \
                                      const T *, T, long, long, long, long, long, T *, int *);         \

@@ -660,6 +660,21 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
     return train_in_place<T>(a_i, a_o, Cij, W, Ci, Cj, nullptr, 0, nullptr, nullptr, B, N, 1, M, taupdt, \
                              cthr, T(0), T(0), T(0));                                                  \
   }                                                                                                    \
+  int sb_update_counters_##SFX(T *Ci, T *Cj, T *Cij, const T *a_i, const T *a_o, T taupdt, long B,     \
+                               long N, long M) {                                                       \
+    SB_READY();                                                                                        \
+    return train_in_place<T>(a_i, a_o, Cij, (T *)nullptr, Ci, Cj, nullptr, 0, nullptr, nullptr, B, N, 1, M, \
+                             taupdt, (T)(taupdt / 2), T(0), T(0), T(0));                               \
+  }                                                                                                    \
+  int sb_weights_from_counters_##SFX(T *W, const T *Ci, const T *Cj, const T *Cij, T cthr, long N,     \
+                                     long M) {                                                         \
+    SB_READY();                                                                                        \
+    return launch_weights_from_traces<T>(g_ctx.stream, W, Ci, Cj, Cij, cthr, N, M);                    \
+  }                                                                                                    \
+  int sb_add_bias_##SFX(T *act, const T *bias, long B, long M) {                                       \
+    SB_READY();                                                                                        \
+    return launch_add_bias<T>(g_ctx.stream, act, bias, B, M);                                          \
+  }                                                                                                    \
   int sb_update_bias_##SFX(T *bias, const T *Cj, T cthr, long M) {                                     \
     SB_READY();                                                                                        \
     return launch_update_bias<T>(g_ctx.stream, bias, Cj, cthr, M);                                     \

@@ -69,7 +69,8 @@ def mask_rows(wmask):
     cap = (int(np.count_nonzero(wmask, axis=0).max(initial=0)) + 15) // 16 * 16 + 16
     d_rows = _dev(np.full((H, cap), -2, dtype=np.int32))
     d_cnt = DeviceArray((H,), np.int32)
-    check(lib().sb_mask_rows(d_rows.ptr, d_cnt.ptr, _dev(wmask).ptr, N, H, cap))
+    d_mask = _dev(wmask)  # kept alive until the results have been copied back
+    check(lib().sb_mask_rows(d_rows.ptr, d_cnt.ptr, d_mask.ptr, N, H, cap))
     return d_rows.numpy(), d_cnt.numpy()
 
 
@@ -78,7 +79,9 @@ def rows_in_blocks(a):
     a = np.ascontiguousarray(a)
     rows, cols = a.shape
     d = DeviceArray(((rows + 15) // 16 * 16 * cols,), a.dtype)
-    check(_fn("sb_rows_in_blocks", a.dtype)(d.ptr, _dev(a).ptr, rows, cols))
+    d_a = _dev(a)  # kept alive until the kernel has run (the stream is synchronised by the next copy)
+    check(_fn("sb_rows_in_blocks", a.dtype)(d.ptr, d_a.ptr, rows, cols))
+    check(lib().sb_sync())
     return d
 
 
@@ -100,7 +103,44 @@ def compute_activation_rows(weights, bias, inputs, wmask, hypercolumns, minicolu
     return d_act.numpy()
 
 
-def update_weights(Ci, Cj, Cij, a_i, a_o, taupdt, weights, cthr):
+def add_bias(a, x):
+    """a[b, :] += x  (kernels_cuda.py:18-26)"""
+    dt = a.dtype
+    B, M = a.shape
+    assert x.shape == (M,)
+    d_a, d_x = _dev(a), _dev(x, dt)
+    check(_fn("sb_add_bias", dt)(d_a.ptr, d_x.ptr, B, M))
+    return _back(a, d_a)
+
+
+def update_counters(Ci, Cj, Cij, a_i, a_o, taupdt):
+    """The trace half of update_weights on its own (kernels_cuda.py:40-48)."""
+    dt = Ci.dtype
+    B, N = a_i.shape
+    M = a_o.shape[1]
+    assert a_o.shape[0] == B and Ci.shape == (N,) and Cj.shape == (M,) and Cij.shape == (N, M)
+    d_ci, d_cj, d_cij = _dev(Ci), _dev(Cj), _dev(Cij)
+    d_x, d_y = _dev(a_i, dt), _dev(a_o, dt)
+    check(_fn("sb_update_counters", dt)(d_ci.ptr, d_cj.ptr, d_cij.ptr, d_x.ptr, d_y.ptr, taupdt, B, N, M))
+    return _back(Ci, d_ci), _back(Cj, d_cj), _back(Cij, d_cij)
+
+
+def update_weights(*args):
+    """Two call forms, told apart by their length:
+    update_weights(Ci, Cj, Cij, a_i, a_o, taupdt, weights, cthr) -- traces and weights in one pass
+        (kernels_openmp.py:18-25); returns (Ci, Cj, Cij, weights);
+    update_weights(weights, Ci, Cj, Cij, cthr) -- the weights from the traces as they are
+        (kernels_cuda.py:51-59); returns weights."""
+    if len(args) == 5:
+        weights, Ci, Cj, Cij, cthr = args
+        dt = weights.dtype
+        N, M = weights.shape
+        assert Ci.shape == (N,) and Cj.shape == (M,) and Cij.shape == (N, M)
+        d_w = DeviceArray((N, M), dt)
+        d_ci, d_cj, d_cij = _dev(Ci, dt), _dev(Cj, dt), _dev(Cij, dt)  # kept alive until the copy back
+        check(_fn("sb_weights_from_counters", dt)(d_w.ptr, d_ci.ptr, d_cj.ptr, d_cij.ptr, cthr, N, M))
+        return _back(weights, d_w)
+    Ci, Cj, Cij, a_i, a_o, taupdt, weights, cthr = args
     dt = Ci.dtype
     f = _fn("sb_update_weights", dt)
     B, N = a_i.shape

@@ -176,6 +176,37 @@ def test_update_weights(k, oracle, dtype, B, N, M):
     assert np.array_equal(g[3] == 0, r[3] == 0)
 
 
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("B,N,M", [(5, 7, 9), (128, 257, 130), (96, 1568, 300), (33, 300, 10)])
+def test_update_counters_then_weights(k, oracle, dtype, B, N, M):
+    """The two halves of update_weights called one after the other (the cuda kernel set's form) give what
+    the fused call gives: traces from update_counters, weights from update_weights(weights, Ci, Cj, Cij,
+    cthr)."""
+    rng = np.random.default_rng(3 * B + N + M)
+    x, y, Ci, Cj, Cij = _trace_problem(rng, B, N, M, dtype)
+    tau = 0.01
+    cthr = tau / 2
+    r = oracle.update_weights(Ci.copy(), Cj.copy(), Cij.copy(), x, y, tau, np.zeros((N, M), dtype=dtype), cthr)
+    ci, cj, cij = k.update_counters(Ci.copy(), Cj.copy(), Cij.copy(), x, y, tau)
+    assert np.array_equal(ci, r[0]) and np.array_equal(cj, r[1])
+    assert_close(cij, r[2], dtype, "Cij")
+    W = k.update_weights(np.full((N, M), 5.0, dtype=dtype), ci, cj, cij, cthr)
+    assert_close(W, r[3], dtype, "W", 2.0)
+    assert np.array_equal(W == 0, r[3] == 0)
+    # and bit for bit what the fused kernel computes from the same traces
+    g = k.update_weights(Ci.copy(), Cj.copy(), Cij.copy(), x, y, tau, np.zeros((N, M), dtype=dtype), cthr)
+    assert np.array_equal(g[2], cij) and np.array_equal(g[3], W)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("B,M", [(1, 1), (7, 33), (128, 3000)])
+def test_add_bias(k, dtype, B, M):
+    rng = np.random.default_rng(B + M)
+    a = rng.standard_normal((B, M)).astype(dtype)
+    b = rng.standard_normal(M).astype(dtype)
+    assert np.array_equal(k.add_bias(a.copy(), b), a + b[None, :])
+
+
 # -------------------------------------------------------------------------------------------- bias
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("M", [1, 10, 3000])
