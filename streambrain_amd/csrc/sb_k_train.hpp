@@ -61,7 +61,8 @@ struct TrainArgs {
   T tau, omt, fB, invB, cthr, cthr4;
   T khalf, pmin, taubdt;
   long tiles_i, tiles_j;
-  FastDiv by_tiles_i, by_Mc;  // divisions by tiles_i and by Mc
+  FastDiv by_panel, by_Mc;  // divisions by tiles_i * panel_cols and by Mc
+  unsigned panel_cols;      // tile order: panels of this many tile columns (a power of two), see the kernel
 };
 
 // MB: mask bytes fetched per vector of VW columns -- 1 when Mc is a multiple of VW (every vector lies
@@ -89,13 +90,25 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, p = lane & 15, q = lane >> 4;
   // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  Renumbered so that one XCD
-  // gets a contiguous run of tiles in column-major order: a few tile columns, i.e. a few hundred KB of
-  // y plus all of x, instead of all of x and y per L2.
+  // gets a contiguous run of tiles.  The run walks the tile grid in panels of panel_cols tile columns,
+  // row by row inside a panel, so the tiles in flight at any time share a few column slabs of y and a
+  // limited set of row slabs of x.  One column per panel (column-major order) when the whole batch of x
+  // fits an L2 anyway: a few hundred KB of y plus all of x per L2.  For big layers a column-major order
+  // re-read x from HBM once per tile column (measured 460 GB per launch at 65536 x 100000, batch 1024).
   const unsigned ntiles = (unsigned)(a.tiles_i * a.tiles_j);  // < 2^31, checked by the launcher
   const unsigned per_xcd = (ntiles + 7) / 8;
   const unsigned tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (tile >= ntiles) return;  // whole workgroup, before any barrier
-  const long jt = a.by_tiles_i.div(tile), it = tile - (unsigned)jt * (unsigned)a.tiles_i;
+  const unsigned panel = a.by_panel.div(tile);
+  const unsigned in_panel = tile - panel * ((unsigned)a.tiles_i * a.panel_cols);
+  long it = in_panel, jt = panel;
+  if (a.panel_cols > 1) {  // uniform
+    const unsigned first = panel * a.panel_cols;
+    const unsigned width = (unsigned)a.tiles_j - first < a.panel_cols ? (unsigned)a.tiles_j - first : a.panel_cols;
+    const unsigned row = width == a.panel_cols ? in_panel >> __builtin_ctz(a.panel_cols) : in_panel / width;
+    it = row;
+    jt = first + (in_panel - row * width);
+  }
   const long i0 = it * TS, j0 = jt * TS;
 
   // thread's share of the tile in row-major order: VW columns of PASSES rows

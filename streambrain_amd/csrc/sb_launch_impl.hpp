@@ -232,7 +232,10 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   a.tau = s.tau; a.omt = s.omt; a.fB = (T)B; a.invB = (T)1 / (T)B; a.cthr = s.cthr; a.cthr4 = s.cthr4;
   a.khalf = khalf; a.pmin = pmin; a.taubdt = taubdt;
   a.tiles_i = cdiv(N, 64); a.tiles_j = cdiv(M, 64);
-  a.by_tiles_i = FastDiv::of(a.tiles_i); a.by_Mc = FastDiv::of(Mc);
+  // tile order (see the kernel): column-major while a batch of x fits an L2 with room to spare, panels of
+  // 8 tile columns beyond that
+  a.panel_cols = B * N * (long)sizeof(T) > (2L << 20) ? 8u : 1u;
+  a.by_panel = FastDiv::of(a.tiles_i * a.panel_cols); a.by_Mc = FastDiv::of(Mc);
   if (M <= 32) {  // a handful of output units: plain vector arithmetic
     const long rows = 256 / M;
     SB_REQUIRE(cdiv(N, rows) < (1L << 31), "too many rows for one launch");
