@@ -74,7 +74,7 @@ def batch_plan(first_step, n_steps, nb):
     return out
 
 
-class GpuRun:
+class DeviceRun:
     def __init__(self, x, y):
         from streambrain_amd import _capi
         self.capi = _capi
@@ -355,7 +355,7 @@ def main():
         return large_workload(args.workload, steps, args.warmup if "--warmup" in sys.argv else nb)
 
     x, y = synthetic_dataset(args.samples)
-    run = GpuRun(x, y)
+    run = DeviceRun(x, y)
 
     run.run_steps(0, args.warmup)
     run.sync()

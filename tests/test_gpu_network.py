@@ -94,6 +94,23 @@ def test_small_network_epochs_with_rewiring_f64(hb, B):
     assert cg.tolist() == cr.tolist() and tg.tolist() == tr.tolist()
 
 
+@pytest.mark.parametrize("n_pix,H,Mc,n_out,Ns,B,density", [
+    (9, 3, 7, 3, 90, 13, 0.5),      # odd everything: minicolumns not a multiple of the vector width
+    (17, 5, 4, 4, 200, 32, 0.2),    # sparse mask, batches of 32 (two row blocks of 16), short last batch
+    (4, 2, 2, 2, 192, 64, 0.5),     # three full batches, two minicolumns
+    (50, 7, 12, 10, 150, 17, 0.15),  # 9 batches, period 1: a rewiring at every step of the later epochs
+    (40, 1, 16, 5, 96, 16, 0.4),    # a single hypercolumn
+])
+def test_odd_shaped_networks_f64(hb, n_pix, H, Mc, n_out, Ns, B, density):
+    # shapes off every tiling's grid, 3 + 2 epochs: whole trajectory in float64, masks included
+    (g, r), (Xt, Yt) = _run_both(hb, np.float64, n_pix=n_pix, H=H, Mc=Mc, n_out=n_out, Ns=Ns, Nt=40, B=B,
+                                 e1=3, e2=2, hp=dict(MNIST_HP, l1_density=density), data_seed=100 + n_pix)
+    assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
+    _compare_states(g, r, 1e-10)
+    assert np.array_equal(g.predict(Xt, B), r.predict(Xt, B))
+    assert rel_err(g.forward(Xt, 7), r.forward(Xt.astype(np.float64))) <= 1e-10
+
+
 def test_small_network_one_epoch_f32(hb):
     # float32, one epoch per layer (13 batches, short last one).  Stated drift bound after one epoch:
     # 1e-4 relative (rounding differences of ~1e-7 per step, amplified by the log of small traces).
