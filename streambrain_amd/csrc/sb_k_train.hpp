@@ -65,10 +65,14 @@ struct TrainArgs {
   unsigned panel_cols;      // tile order: panels of this many tile columns (a power of two), see the kernel
 };
 
+#ifndef SB_TRAIN_WAVES
+#define SB_TRAIN_WAVES(T) sizeof(T) == 8 ? 4 : 5
+#endif
 // MB: mask bytes fetched per vector of VW columns -- 1 when Mc is a multiple of VW (every vector lies
 // inside one hypercolumn), VW otherwise.
 template <typename T, int KCH, bool VEC, int MB>
-__global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SB_TRAIN_WAVES(T))))
+void k_train_fused(TrainArgs<T> a) {
   using R = Real<T>;
   using acc_t = typename R::acc_t;
   constexpr int VW = R::VW;             // elements per 16-byte vector
@@ -78,6 +82,13 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   constexpr int PASSES = TS / RPP;      // passes over the tile (epilogue, Cij prefetch)
   constexpr int SP = KCH / RPP;         // staging passes per chunk
   constexpr int CP = TS + VW;           // pitch of the accumulator tile in LDS
+  // A staged slab row of 64 floats spans the 64 LDS banks exactly, and an 8-byte operand read is served
+  // 32 lanes at a time: lanes (p, q) and (p, q+1), one slab row apart, would meet in the same banks.  Odd
+  // slab rows therefore hold their two halves swapped (column ^ 32).  16-byte reads (doubles) are served
+  // 16 lanes at a time, one slab row: nothing to do.
+  constexpr int SWZ = sizeof(T) == 4 ? 32 : 0;
+  constexpr bool TILE_IN_LAST = sizeof(T) == 8;  // which chunk requests the Cij tile, see the chunk loop
+  static_assert(RPP % 2 == 0, "row parity of a staging pass");
   static_assert(KCH % RPP == 0 && KCH % 4 == 0, "chunk size");
   // LDS: the staging slabs xs | ys; once they are consumed the same memory holds the accumulator tile
   // followed by the trace reciprocals of the tile's rows and columns
@@ -151,7 +162,7 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
   const bool summer = role < 2;  // uniform per wavefront
   const bool sum_i = role == 0;
   const int scol = lane;
-  const T *sbase = (sum_i ? xs : ys) + scol;
+  const T *sbase = (sum_i ? xs : ys) + scol, *sbase_odd = (sum_i ? xs : ys) + (scol ^ SWZ);
   const long sidx = (sum_i ? i0 : j0) + scol;
   const bool sum_ok = summer && sidx < (sum_i ? a.N : a.M);
   const bool writes_bias = sum_ok && !sum_i && it == 0 && a.bias_mode == 1;
@@ -204,8 +215,9 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
         vx[e] = sx[m][e];
         vy[e] = sy[m][e];
       }
-      *reinterpret_cast<typename R::vec_t *>(&xs[(er + RPP * m) * TS + VW * eg]) = vx;
-      *reinterpret_cast<typename R::vec_t *>(&ys[(er + RPP * m) * TS + VW * eg]) = vy;
+      const int at = (er + RPP * m) * TS + ((VW * eg) ^ ((er & 1) * SWZ));
+      *reinterpret_cast<typename R::vec_t *>(&xs[at]) = vx;
+      *reinterpret_cast<typename R::vec_t *>(&ys[at]) = vy;
     }
     __syncthreads();
     SB_PHASE_MARK(1 + 2 * (int)(b0 / KCH));
@@ -218,7 +230,7 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
       for (int r = 0; r < KCH; r += 16) {
         T v[16];
 #pragma unroll
-        for (int k = 0; k < 16; k++) v[k] = sbase[(r + k) * TS];
+        for (int k = 0; k < 16; k++) v[k] = (k & 1 ? sbase_odd : sbase)[(r + k) * TS];
 #pragma unroll
         for (int k = 0; k < 16; k++) csum = R::add(csum, v[k]);
       }
@@ -226,8 +238,8 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
 
     // K loop: per step of 4 batch rows, lane (p,q) feeds row 4s+q of the slabs.  The operands of step
     // s+1 are read from LDS before the MFMAs of step s are issued (the fences keep that order).
-    const T *xa = xs + q * TS + iw + 2 * p;
-    const T *ya = ys + q * TS + jw + 2 * p;
+    const T *xa = xs + q * TS + ((iw + 2 * p) ^ ((q & 1) * SWZ));
+    const T *ya = ys + q * TS + ((jw + 2 * p) ^ ((q & 1) * SWZ));
     T xo[2][2], yo[2][2];
     xo[0][0] = xa[0], xo[0][1] = xa[1], yo[0][0] = ya[0], yo[0][1] = ya[1];
 #pragma unroll
@@ -246,10 +258,17 @@ __global__ __launch_bounds__(256) void k_train_fused(TrainArgs<T> a) {
     }
   };
   long b0 = 0;
-  for (; b0 + 2 * KCH < a.B; b0 += KCH) chunk(b0, std::false_type{});
-  chunk(b0, std::true_type{});  // second-to-last (or only) chunk: the Cij tile is requested here
-  b0 += KCH;
-  if (b0 < a.B) chunk(b0, std::false_type{});
+  if constexpr (TILE_IN_LAST) {
+    // doubles: a chunk takes twice as long, enough to cover the tile's latency, and the tile's registers
+    // then never coexist with the staging registers of a further chunk
+    for (; b0 + KCH < a.B; b0 += KCH) chunk(b0, std::false_type{});
+    chunk(b0, std::true_type{});
+  } else {
+    for (; b0 + 2 * KCH < a.B; b0 += KCH) chunk(b0, std::false_type{});
+    chunk(b0, std::true_type{});  // second-to-last (or only) chunk: the Cij tile is requested here
+    b0 += KCH;
+    if (b0 < a.B) chunk(b0, std::false_type{});
+  }
 
   __syncthreads();  // slabs consumed: their memory is reused from here on
   SB_PHASE_MARK(12);
