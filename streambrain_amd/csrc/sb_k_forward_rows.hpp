@@ -22,6 +22,21 @@ struct ForwardRowsArgs {
   const T *xt;         // XT kernels: the batch in blocks of 16 rows (k_gather_rows_blocked), from row 0
 };
 
+// Wavefronts per SIMD the kernel's registers are budgeted for: three or two (as many workgroups of four
+// wavefronts per CU, one computing while another waits for its gathers) where the operand ring, the
+// accumulators and the x operands leave room for that, one for the big tiles.
+template <typename T, int NG>
+constexpr int forward_rows_regs(int rb) {  // registers of the three, in 32-bit units
+  constexpr int VW = Real<T>::VW, D = sizeof(T) / 4;
+  return (2 * VW * NG * VW + rb * NG * VW * 4 + 2 * rb * VW) * D;
+}
+constexpr int kRowsRegsTwoWaves = 150, kRowsRegsThreeWaves = 104;  // measured: no spills up to these
+template <typename T, int NG, int RB>
+constexpr int forward_rows_waves_per_simd() {
+  constexpr int regs = forward_rows_regs<T, NG>(RB);
+  return regs <= kRowsRegsThreeWaves ? 3 : regs <= kRowsRegsTwoWaves ? 2 : 1;
+}
+
 // A workgroup owns 16 batch rows x one hypercolumn (as k_forward with FUSE).  The hypercolumn's row list
 // is staged through LDS in segments of SEG entries; the wavefronts split a segment in interleaved chunks
 // of 4*VW entries.  Per chunk, lane (p,q) reads the VW list entries VW*q .. VW*q+VW-1 from LDS, then
@@ -37,7 +52,8 @@ struct ForwardRowsArgs {
 // consecutive elements (one 64-byte access) instead of one element each of 16 rows.
 template <typename T, int NG, int NWAVES, int RB = 1, bool XT = false>
 __global__ __launch_bounds__(64 * NWAVES)
-__attribute__((amdgpu_waves_per_eu(NWAVES >= 4 ? NWAVES / 4 : 1, NWAVES >= 4 ? NWAVES / 4 : 1)))
+__attribute__((amdgpu_waves_per_eu(forward_rows_waves_per_simd<T, NG, RB>(),
+                                   forward_rows_waves_per_simd<T, NG, RB>())))
 void k_forward_rows(ForwardRowsArgs<T> ar) {
   const ForwardArgs<T> &a = ar.f;
   constexpr int VW = Real<T>::VW;
