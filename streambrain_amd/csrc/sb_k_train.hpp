@@ -65,13 +65,14 @@ struct TrainArgs {
   unsigned panel_cols;      // tile order: panels of this many tile columns (a power of two), see the kernel
 };
 
-#ifndef SB_TRAIN_WAVES
-#define SB_TRAIN_WAVES(T) sizeof(T) == 8 ? 4 : 5
-#endif
+// Wavefronts per SIMD the registers are budgeted for.  Doubles: four (the LDS slabs allow four workgroups
+// per CU; left alone the compiler takes 176 registers, which allows two).  Floats need no limit: 80-96.
+template <typename T>
+constexpr int train_waves_per_simd() { return sizeof(T) == 8 ? 4 : 1; }
 // MB: mask bytes fetched per vector of VW columns -- 1 when Mc is a multiple of VW (every vector lies
 // inside one hypercolumn), VW otherwise.
 template <typename T, int KCH, bool VEC, int MB>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SB_TRAIN_WAVES(T))))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(train_waves_per_simd<T>())))
 void k_train_fused(TrainArgs<T> a) {
   using R = Real<T>;
   using acc_t = typename R::acc_t;
