@@ -118,13 +118,7 @@ __global__ __launch_bounds__(256) void k_train_skinny(TrainArgs<T> a) {
       sy = Rl::add(sy, yk);
     }
   }
-  auto trace = [&](T cold, T sum) {
-    T s = Rl::div(sum, a.fB);
-    s = Rl::mul(s, a.tau);
-    const T c = Rl::add(Rl::mul(cold, a.omt), s);
-    return c > T(0) ? c : T(0);
-  };
-  const T ci = trace(a.Ci[i], sx), cj = trace(a.Cj[j], sy);
+  const T ci = trace_next<T>(a.Ci[i], sx, a), cj = trace_next<T>(a.Cj[j], sy, a);
   if (j == 0) a.Ci_next[i] = ci;
   if (i == 0) {
     a.Cj_next[j] = cj;

@@ -65,13 +65,61 @@ struct TrainArgs {
   unsigned panel_cols;      // tile order: panels of this many tile columns (a power of two), see the kernel
 };
 
+// New trace from the old one and the batch's column sum, in the reference's order of operations
+// (kernels_openmp_internal.cc:117-129): sum / B, times tau, plus old * (1 - tau), clamped at 0.
+template <typename T>
+__device__ inline T trace_next(T cold, T sum, const TrainArgs<T> &a) {
+  using R = Real<T>;
+  T s = R::div(sum, a.fB);
+  s = R::mul(s, a.tau);
+  const T c = R::add(R::mul(cold, a.omt), s);
+  return c > T(0) ? c : T(0);
+}
+
+// The new traces Ci_next, Cj_next (and the regularized bias) on their own, a thread per input or output
+// unit walking the batch in order: what every tile of k_train_fused otherwise repeats for its own 64 rows
+// and 64 columns.  Launched ahead of k_train_fused<.., PRE = true> when a layer has so many tiles that the
+// repetition costs more than a launch.
+template <typename T>
+__global__ __launch_bounds__(256) void k_trace_sums(TrainArgs<T> a) {
+  using R = Real<T>;
+  const long t = (long)blockIdx.x * 256 + threadIdx.x;
+  const bool is_i = t < a.N;
+  const long idx = is_i ? t : t - a.N;
+  if (!is_i && idx >= a.M) return;
+  const T *p = (is_i ? a.x : a.y) + idx;
+  const long stride = is_i ? a.N : a.M;
+  T sum = T(0);
+  long b = 0;
+  for (; b + 16 <= a.B; b += 16) {  // 16 loads in flight, then the ordered additions
+    T v[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) v[k] = p[(b + k) * stride];
+#pragma unroll
+    for (int k = 0; k < 16; k++) sum = R::add(sum, v[k]);
+  }
+  for (; b < a.B; b++) sum = R::add(sum, p[b * stride]);
+  const T cnew = trace_next<T>((is_i ? a.Ci : a.Cj)[idx], sum, a);
+  if (is_i) {
+    a.Ci_next[idx] = cnew;
+  } else {
+    a.Cj_next[idx] = cnew;
+    if (a.bias_mode == 1) {
+      T kb = a.kbi[idx];
+      a.bias[idx] = bias_regularized<T>(cnew, kb, a.cthr, a.khalf, a.pmin, a.taubdt);
+      a.kbi[idx] = kb;
+    }
+  }
+}
+
 // Wavefronts per SIMD the registers are budgeted for.  Doubles: four (the LDS slabs allow four workgroups
 // per CU; left alone the compiler takes 176 registers, which allows two).  Floats need no limit: 80-96.
 template <typename T>
 constexpr int train_waves_per_simd() { return sizeof(T) == 8 ? 4 : 1; }
 // MB: mask bytes fetched per vector of VW columns -- 1 when Mc is a multiple of VW (every vector lies
 // inside one hypercolumn), VW otherwise.
-template <typename T, int KCH, bool VEC, int MB>
+// PRE: Ci_next and Cj_next already hold the new traces (k_trace_sums): no column sums here.
+template <typename T, int KCH, bool VEC, int MB, bool PRE = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(train_waves_per_simd<T>())))
 void k_train_fused(TrainArgs<T> a) {
   using R = Real<T>;
@@ -166,10 +214,11 @@ void k_train_fused(TrainArgs<T> a) {
   const T *sbase = (sum_i ? xs : ys) + scol, *sbase_odd = (sum_i ? xs : ys) + (scol ^ SWZ);
   const long sidx = (sum_i ? i0 : j0) + scol;
   const bool sum_ok = summer && sidx < (sum_i ? a.N : a.M);
-  const bool writes_bias = sum_ok && !sum_i && it == 0 && a.bias_mode == 1;
-  const T cold = (sum_i ? a.Ci : a.Cj)[sum_ok ? sidx : 0];  // old trace
+  const bool writes_bias = !PRE && sum_ok && !sum_i && it == 0 && a.bias_mode == 1;
+  // old trace; with PRE the new one, which the same two wavefronts turn into the reciprocals below
+  const T cold = (PRE ? (sum_i ? a.Ci_next : a.Cj_next) : (sum_i ? a.Ci : a.Cj))[sum_ok ? sidx : 0];
   T kb = T(1);
-  if (a.bias_mode == 1) kb = a.kbi[writes_bias ? sidx : 0];
+  if (!PRE && a.bias_mode == 1) kb = a.kbi[writes_bias ? sidx : 0];
   T csum = T(0);
 
   // mask bytes of the thread's PASSES x VW synapses: a small, L2-resident array, fetched up front
@@ -225,7 +274,7 @@ void k_train_fused(TrainArgs<T> a) {
     request_chunk(b0 + KCH);  // past the batch: reads zeros nobody consumes
     if (decltype(with_tile)::value) request_tile();
 
-    if (summer) {
+    if (!PRE && summer) {
       // rows past the end of the batch were staged as zeros: adding them changes nothing, so the loop
       // needs no guard; 16 LDS reads are in flight before the (ordered) additions consume them
       for (int r = 0; r < KCH; r += 16) {
@@ -278,17 +327,18 @@ void k_train_fused(TrainArgs<T> a) {
   if (summer) {
     T cnew = T(1);
     if (sum_ok) {
-      T s = R::div(csum, a.fB);
-      s = R::mul(s, a.tau);
-      cnew = R::add(R::mul(cold, a.omt), s);
-      cnew = cnew > T(0) ? cnew : T(0);
-      if (sum_i) {
-        if (jt == 0) a.Ci_next[sidx] = cnew;
-      } else if (it == 0) {
-        a.Cj_next[sidx] = cnew;
-        if (writes_bias) {
-          a.bias[sidx] = bias_regularized<T>(cnew, kb, a.cthr, a.khalf, a.pmin, a.taubdt);
-          a.kbi[sidx] = kb;
+      if constexpr (PRE) {
+        cnew = cold;
+      } else {
+        cnew = trace_next<T>(cold, csum, a);
+        if (sum_i) {
+          if (jt == 0) a.Ci_next[sidx] = cnew;
+        } else if (it == 0) {
+          a.Cj_next[sidx] = cnew;
+          if (writes_bias) {
+            a.bias[sidx] = bias_regularized<T>(cnew, kb, a.cthr, a.khalf, a.pmin, a.taubdt);
+            a.kbi[sidx] = kb;
+          }
         }
       }
     }

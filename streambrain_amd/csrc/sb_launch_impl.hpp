@@ -260,7 +260,13 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   constexpr int KCH = 32;
   const bool one_byte = Mc % VW == 0;  // every vector of VW columns lies inside one hypercolumn
   ProfScope prof_(st, K_TRAIN_FUSED);
-  if (vec && one_byte)
+  // Every tile adds up the batch's x and y columns for its own rows and columns, which with many tile
+  // rows and columns is most of the kernel's vector arithmetic (43 % at 65536 x 100000, batch 1024).
+  // From 16 rounds of workgroups on, a small launch computes the new traces once and the tiles read them.
+  if (vec && one_byte && a.tiles_i * a.tiles_j >= 16 * 5 * device_cu_count()) {
+    hipLaunchKernelGGL((k_trace_sums<T>), dim3((unsigned)cdiv(N + M, 256)), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((k_train_fused<T, KCH, true, 1, true>), grid, dim3(256), 0, st, a);
+  } else if (vec && one_byte)
     hipLaunchKernelGGL((k_train_fused<T, KCH, true, 1>), grid, dim3(256), 0, st, a);
   else if (vec)
     hipLaunchKernelGGL((k_train_fused<T, KCH, true, VW>), grid, dim3(256), 0, st, a);

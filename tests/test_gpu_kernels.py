@@ -162,7 +162,9 @@ def _trace_problem(rng, B, N, M, dtype):
 @pytest.mark.parametrize("B,N,M", SHAPES + [(128, 1568, 3000), (5, 130, 70), (1024, 64, 64),
                                            # batch of x above 2 MiB: tiles walked in panels of 8 tile
                                            # columns; 11 and 8 tile columns (narrow and no last panel)
-                                           (64, 8300, 700), (48, 5600, 512)])
+                                           (64, 8300, 700), (48, 5600, 512),
+                                           # 150 x 141 tiles: the traces come from their own launch
+                                           (8, 9600, 9000)])
 def test_update_weights(k, oracle, dtype, B, N, M):
     rng = np.random.default_rng(B + 2 * N + 3 * M)
     x, y, Ci, Cj, Cij = _trace_problem(rng, B, N, M, dtype)
