@@ -95,10 +95,11 @@ int launch_forward_classify(hipStream_t st, T *act, const T *x, const T *W, cons
       constexpr int NGL = 8 / VW, LWL = 7 - (NGL - 1) * VW;  // float: 2 groups, 3 blocks; double: 4, 1
       if ((Mc - (NGL - 1) * GW) % LWL == 0) {
         // Large batches: 64 or 32 rows per workgroup instead of 16 while there still are enough tiles for
-        // eight / four rounds of workgroups, so that W crosses the L2 -> L1 path a quarter / half as often.
+        // eight rounds / one round of workgroups, so that W crosses the L2 -> L1 path a quarter / half as
+        // often (64 rows with fewer rounds lose more to the last, partly filled round than they gain).
         const long cus = device_cu_count();
         // (double: at most 32 rows, 64 do not fit the register file)
-        long rb = sizeof(T) == 4 && H * cdiv(B, 64) >= 8 * cus ? 4 : (H * cdiv(B, 32) >= 4 * cus ? 2 : 1);
+        long rb = sizeof(T) == 4 && H * cdiv(B, 64) >= 8 * cus ? 4 : (H * cdiv(B, 32) >= cus ? 2 : 1);
         // (32-bit byte offsets inside the tile's rows)
         while (rb > 1 && 16 * rb * N * (long)sizeof(T) >= (1L << 31)) rb /= 2;
         a.batch_tiles = cdiv(B, 16 * rb);
@@ -145,13 +146,13 @@ static int forward_rows_variant(hipStream_t st, ForwardRowsArgs<T> a) {
   ProfScope prof_(st, K_FORWARD);
   // four wavefronts measured best (8: 8.8 us, 4: 8.2 us, 2: 9.9 us, 16: 10.7 us at 1568 -> 30x100, density 0.1)
   constexpr int NW = 4;
-  // large batches: 64 or 32 rows per workgroup while there are tiles for eight / four rounds of
-  // workgroups (as in launch_forward), as long as the kernel then still fits two wavefronts per SIMD:
+  // large batches: 64 or 32 rows per workgroup while there are tiles for eight rounds / three quarters
+  // of a round of workgroups (much as in launch_forward), as long as the kernel then still fits two wavefronts per SIMD:
   // two workgroups per CU with fewer rows each beat one with more (204 against 240 us at 1568 -> 30x100,
   // batch 8192; 70 against 83 us at 1568 -> 100x100 in double, batch 512)
   const long cus = device_cu_count(), H = a.f.col_tiles, B = a.f.B;
   constexpr bool fits4 = forward_rows_regs<T, NG>(4) <= kRowsRegsTwoWaves;
-  long rb = fits4 && H * cdiv(B, 64) >= 8 * cus ? 4 : (H * cdiv(B, 32) >= 4 * cus ? 2 : 1);
+  long rb = fits4 && H * cdiv(B, 64) >= 8 * cus ? 4 : (4 * H * cdiv(B, 32) >= 3 * cus ? 2 : 1);
   while (rb > 1 && forward_rows_regs<T, NG>((int)rb) > kRowsRegsTwoWaves) rb /= 2;
   // (32-bit byte offsets inside the tile's rows)
   while (rb > 1 && 16 * rb * a.f.N * (long)sizeof(T) >= (1L << 31)) rb /= 2;
