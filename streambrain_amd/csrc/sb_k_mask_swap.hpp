@@ -1,6 +1,6 @@
 // Register-resident variant of the greedy swap loop of the mask rewiring (omp.cc:289-315, where
 // "omp.cc" = BCPNN/backend/_kernels/kernels_openmp_internal.cc of the reference) for layers with at
-// most NT*R input rows: one small workgroup of NT threads, thread t owns rows t, t+NT, ...; score
+// most NT*R input rows: one workgroup of NT threads, thread t owns rows t, t+NT, ...; score
 // nominators, connection counts, mask bits and scores stay in registers over all iterations.  Per
 // iteration: a DPP / shuffle reduction inside each wavefront, one partial result per wavefront through
 // LDS, a second reduction that leaves the decision in every lane -- one barrier.  Same decisions as
@@ -161,8 +161,10 @@ struct MaskSwapFast {
   using SK = ScoreKey<T>;
   using K = typename SK::K;
   static constexpr int TOPK = 16, CAP = 48, DIG = 11, BINS = 1 << DIG, PER = BINS / NT, NWV = NT / 64;
-  static constexpr int ISH = NT * R > BINS ? 2 : 0;  // index bins of the tie cut: (row index) >> ISH
-  static_assert(NT * R <= (BINS << 2) && BINS % NT == 0, "row indices must fit the index histogram");
+  // index bins of the tie cut: (row index) >> ISH, the smallest shift that fits NT * R rows into BINS bins
+  static constexpr int ish_for(int rows) { return rows <= BINS ? 0 : 1 + ish_for((rows + 1) / 2); }
+  static constexpr int ISH = ish_for(NT * R);
+  static_assert(((NT * R - 1) >> ISH) < BINS && BINS % NT == 0, "row indices must fit the index histogram");
   struct Shared {
     unsigned hist[2][BINS];
     int cand[2][64], cand_cs[2][64];  // candidate rows, their connection counts ...
@@ -364,12 +366,12 @@ struct MaskSwapFast {
   }
 };
 
-// NT threads (a multiple of 64, at most 256: one wavefront per SIMD, so the replicated reduction code
-// is not time-shared), thread t owns rows t, t+NT, ..., t+(R-1)*NT.
+// NT threads (64 to 1024 in powers of two), thread t owns rows t, t+NT, ..., t+(R-1)*NT.  1024 threads
+// with few rows each measured faster than 256 with more (1568 rows: 19.8 against 21.8 us).
 template <typename T, int NT, int R>
 __global__ __launch_bounds__(NT) void k_mask_swap_reg(MaskArgs<T> a) {
   constexpr int NWV = NT / 64;
-  static_assert(NWV == 1 || NWV == 2 || NWV == 4, "1, 2 or 4 wavefronts");
+  static_assert(NWV == 1 || NWV == 2 || NWV == 4 || NWV == 8 || NWV == 16, "1 to 16 wavefronts");
   __shared__ RowCand<T> part[2][4][NWV];  // [buffer][max0, min1, first0, first1][wavefront]
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
 
@@ -455,6 +457,18 @@ __global__ __launch_bounds__(NT) void k_mask_swap_reg(MaskArgs<T> a) {
         cmin = pick_min<T>(cmin, dpp_cand<kDppSwap2, T>(cmin));
         f0 = pick_first<T>(f0, dpp_cand<kDppSwap2, T>(f0));
         f1 = pick_first<T>(f1, dpp_cand<kDppSwap2, T>(f1));
+      }
+      if (NWV > 4) {  // the lanes of a quad agree by now, so mirroring 8 (16) lanes pairs the quads
+        cmax = pick_max<T>(cmax, dpp_cand<kDppHalfMirror, T>(cmax));
+        cmin = pick_min<T>(cmin, dpp_cand<kDppHalfMirror, T>(cmin));
+        f0 = pick_first<T>(f0, dpp_cand<kDppHalfMirror, T>(f0));
+        f1 = pick_first<T>(f1, dpp_cand<kDppHalfMirror, T>(f1));
+      }
+      if (NWV > 8) {
+        cmax = pick_max<T>(cmax, dpp_cand<kDppMirror, T>(cmax));
+        cmin = pick_min<T>(cmin, dpp_cand<kDppMirror, T>(cmin));
+        f0 = pick_first<T>(f0, dpp_cand<kDppMirror, T>(f0));
+        f1 = pick_first<T>(f1, dpp_cand<kDppMirror, T>(f1));
       }
     }
     if (cmax.idx < 0 && f0.idx < 0) break;  // no silent row (uniform over the workgroup)

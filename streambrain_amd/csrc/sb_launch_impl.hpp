@@ -350,9 +350,13 @@ int launch_update_mask(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, 
   if (iterations > 0) {
     ProfScope prof_(st, K_MASK_SWAP);
     if (N <= 2048)
-      hipLaunchKernelGGL((k_mask_swap_reg<T, 256, 8>), dim3(1), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_mask_swap_reg<T, 1024, 2>), dim3(1), dim3(1024), 0, st, a);
     else if (N <= 8192)
-      hipLaunchKernelGGL((k_mask_swap_reg<T, 256, 32>), dim3(1), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_mask_swap_reg<T, 1024, 8>), dim3(1), dim3(1024), 0, st, a);
+    else if (N <= 32768)
+      hipLaunchKernelGGL((k_mask_swap_reg<T, 1024, 32>), dim3(1), dim3(1024), 0, st, a);
+    else if (N <= 65536)
+      hipLaunchKernelGGL((k_mask_swap_reg<T, 1024, 64>), dim3(1), dim3(1024), 0, st, a);
     else
       hipLaunchKernelGGL((k_mask_swap<T>), dim3(1), dim3(1024), 0, st, a);
     SB_LAUNCH_CHECK();

@@ -248,7 +248,8 @@ def _mask_problem(rng, N, H, Mc, dtype, density=0.1):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("N,H,Mc", [(1, 1, 2), (7, 2, 3), (128, 5, 20), (1568, 30, 100), (5000, 3, 4), (9000, 2, 3)])
+@pytest.mark.parametrize("N,H,Mc", [(1, 1, 2), (7, 2, 3), (128, 5, 20), (1568, 30, 100), (5000, 3, 4), (9000, 2, 3),
+                                    (20000, 2, 3), (40000, 2, 3), (70000, 1, 2)])
 @pytest.mark.parametrize("iterations", [0, 1, 16])
 def test_update_mask_bit_exact(k, oracle, dtype, N, H, Mc, iterations):
     rng = np.random.default_rng(N + H + Mc)
@@ -277,7 +278,7 @@ def test_update_mask_ties_and_degenerate_columns(k, oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("N,H,Mc", [(1568, 30, 100), (300, 4, 10), (6000, 3, 8)])
+@pytest.mark.parametrize("N,H,Mc", [(1568, 30, 100), (300, 4, 10), (6000, 3, 8), (12000, 2, 4), (50000, 2, 4)])
 @pytest.mark.parametrize("kind", ["dead_rows", "near_equal", "identical_rows", "few_active", "few_silent"])
 def test_update_mask_tie_blocks(k, oracle, dtype, N, H, Mc, kind):
     """Score distributions that stress the candidate preselection of the swap loop: large blocks of
