@@ -34,7 +34,6 @@ struct Context {
   // scratch of the per-kernel training entry points: the "next" Ci / Cj of the fused kernel
   void *trace_next = nullptr;
   long trace_cap = 0;  // elements of 8 bytes
-  // partial sums of the split-K forward, shared by every caller (stream order serialises its use)
 };
 static Context g_ctx;
 static std::mutex g_ctx_mutex;
@@ -184,6 +183,17 @@ struct sb_net {
 namespace sb {
 
 static inline long cdiv_l(long a, long b) { return (a + b - 1) / b; }
+
+// Device allocation that is released when the scope ends, whichever way it ends.
+struct ScopedDeviceBuffer {
+  void *p = nullptr;
+  ScopedDeviceBuffer() = default;
+  ScopedDeviceBuffer(const ScopedDeviceBuffer &) = delete;
+  ScopedDeviceBuffer &operator=(const ScopedDeviceBuffer &) = delete;
+  ~ScopedDeviceBuffer() {
+    if (p) (void)hipFree(p);
+  }
+};
 
 static int free_dev(void *&p) {
   if (p) SB_HIP(hipFree(p));
@@ -356,35 +366,35 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
   const bool permute = first_batch == 0;  // a later range continues the epoch already laid out
   SB_REQUIRE(permute || net->Xp, "the epoch's first batches have not been run");
   if (permute) {
-  SB_REQUIRE(h_sample_perm, "sample order missing");
-  for (long r = 0; r < Ns; r++)
-    SB_REQUIRE(h_sample_perm[r] >= 0 && h_sample_perm[r] < Ns, "sample index out of range");
+    SB_REQUIRE(h_sample_perm, "sample order missing");
+    for (long r = 0; r < Ns; r++)
+      SB_REQUIRE(h_sample_perm[r] >= 0 && h_sample_perm[r] < Ns, "sample index out of range");
 
-  // images[idx, :] / labels[idx, :]  (_cpu_base_backend.py:258-260)
-  if (!net->Xp) SB_HIP(hipMalloc(&net->Xp, (size_t)Ns * net->NF * net->esize));
-  if (last && !net->Yp) SB_HIP(hipMalloc(&net->Yp, (size_t)Ns * net->NC * net->esize));
-  SB_HIP(hipEventSynchronize(net->perm_copied));  // staging buffer free again
-  std::memcpy(net->h_perm, h_sample_perm, (size_t)Ns * sizeof(int64_t));
-  SB_HIP(hipMemcpyAsync(net->d_perm, net->h_perm, (size_t)Ns * sizeof(int64_t), hipMemcpyHostToDevice,
-                        st));
-  SB_HIP(hipEventRecord(net->perm_copied, st));
-  // A first layer that walks row lists reads its input column by column: it gets the shuffled images a
-  // second time, in blocks of 16 rows (batches must then start on block boundaries); one kernel writes
-  // both copies from one read.
-  if (net->layers[0].rows && maxB % 16 == 0) {
-    if (!net->XpB) SB_HIP(hipMalloc(&net->XpB, (size_t)cdiv_l(Ns, 16) * 16 * net->NF * net->esize));
-    if ((rc = launch_gather_rows_blocked<T>(st, (T *)net->XpB, (T *)net->Xp, (const T *)net->X, net->d_perm, Ns,
-                                            net->NF)))
-      return rc;
-    net->XpB_batch = maxB;
-  } else {
-    if ((rc = launch_gather_rows<T>(st, (T *)net->Xp, (const T *)net->X, net->d_perm, Ns, net->NF)))
-      return rc;
-    net->XpB_batch = 0;
-  }
-  if (last)
-    if ((rc = launch_gather_rows<T>(st, (T *)net->Yp, (const T *)net->Y, net->d_perm, Ns, net->NC)))
-      return rc;
+    // images[idx, :] / labels[idx, :]  (_cpu_base_backend.py:258-260)
+    if (!net->Xp) SB_HIP(hipMalloc(&net->Xp, (size_t)Ns * net->NF * net->esize));
+    if (last && !net->Yp) SB_HIP(hipMalloc(&net->Yp, (size_t)Ns * net->NC * net->esize));
+    SB_HIP(hipEventSynchronize(net->perm_copied));  // staging buffer free again
+    std::memcpy(net->h_perm, h_sample_perm, (size_t)Ns * sizeof(int64_t));
+    SB_HIP(hipMemcpyAsync(net->d_perm, net->h_perm, (size_t)Ns * sizeof(int64_t), hipMemcpyHostToDevice,
+                          st));
+    SB_HIP(hipEventRecord(net->perm_copied, st));
+    // A first layer that walks row lists reads its input column by column: it gets the shuffled images a
+    // second time, in blocks of 16 rows (batches must then start on block boundaries); one kernel writes
+    // both copies from one read.
+    if (net->layers[0].rows && maxB % 16 == 0) {
+      if (!net->XpB) SB_HIP(hipMalloc(&net->XpB, (size_t)cdiv_l(Ns, 16) * 16 * net->NF * net->esize));
+      if ((rc = launch_gather_rows_blocked<T>(st, (T *)net->XpB, (T *)net->Xp, (const T *)net->X, net->d_perm, Ns,
+                                              net->NF)))
+        return rc;
+      net->XpB_batch = maxB;
+    } else {
+      if ((rc = launch_gather_rows<T>(st, (T *)net->Xp, (const T *)net->X, net->d_perm, Ns, net->NF)))
+        return rc;
+      net->XpB_batch = 0;
+    }
+    if (last)
+      if ((rc = launch_gather_rows<T>(st, (T *)net->Yp, (const T *)net->Y, net->d_perm, Ns, net->NC)))
+        return rc;
   }
 
   const long period = nb / (target.H + 1);  // _cpu_base_backend.py:297-299
@@ -443,14 +453,15 @@ static int net_forward_batches(sb_net *net, const void *h_images, const void *h_
   chunk = chunk / maxB * maxB;
   if (chunk < maxB) chunk = maxB;
   if (chunk > n) chunk = n;
-  void *dX = nullptr, *dY = nullptr, *dXB = nullptr;
-  int32_t *dP = nullptr;
-  SB_HIP(hipMalloc(&dX, (size_t)chunk * NF * sizeof(T)));
+  ScopedDeviceBuffer bX, bY, bXB, bP;
+  SB_HIP(hipMalloc(&bX.p, (size_t)chunk * NF * sizeof(T)));
   // a first layer that walks row lists also gets every chunk in blocks of 16 rows (see net_train_batches)
   const bool blocked = net->layers[0].rows && maxB % 16 == 0;
-  if (blocked) SB_HIP(hipMalloc(&dXB, (size_t)cdiv_l(chunk, 16) * 16 * NF * sizeof(T)));
-  if (h_labels) SB_HIP(hipMalloc(&dY, (size_t)chunk * NC * sizeof(T)));
-  if (h_pred) SB_HIP(hipMalloc((void **)&dP, (size_t)chunk * sizeof(int32_t)));
+  if (blocked) SB_HIP(hipMalloc(&bXB.p, (size_t)cdiv_l(chunk, 16) * 16 * NF * sizeof(T)));
+  if (h_labels) SB_HIP(hipMalloc(&bY.p, (size_t)chunk * NC * sizeof(T)));
+  if (h_pred) SB_HIP(hipMalloc(&bP.p, (size_t)chunk * sizeof(int32_t)));
+  void *const dX = bX.p, *const dY = bY.p, *const dXB = bXB.p;
+  int32_t *const dP = (int32_t *)bP.p;
   if (h_labels) {
     unsigned long long zero = 0;
     SB_HIP(hipMemcpy(net->d_correct, &zero, sizeof(zero), hipMemcpyHostToDevice));
@@ -497,10 +508,7 @@ static int net_forward_batches(sb_net *net, const void *h_images, const void *h_
     SB_HIP(hipMemcpy(&cnt, net->d_correct, sizeof(cnt), hipMemcpyDeviceToHost));
     *correct = (int64_t)cnt;
   }
-  SB_HIP(hipFree(dX));
-  if (dXB) SB_HIP(hipFree(dXB));
-  if (dY) SB_HIP(hipFree(dY));
-  if (dP) SB_HIP(hipFree(dP));
+  if (rc) (void)hipStreamSynchronize(st);  // nothing in flight may still use the chunk buffers
   return rc;
 }
 
@@ -738,6 +746,8 @@ int sb_net_create(sb_net **net, int dtype) {
   if (e == hipSuccess) e = hipMalloc((void **)&n->d_unmasked, sizeof(unsigned long long));
   if (e == hipSuccess) e = hipEventCreateWithFlags(&n->perm_copied, hipEventDisableTiming);
   if (e != hipSuccess) {
+    if (n->d_correct) (void)hipFree(n->d_correct);
+    if (n->d_unmasked) (void)hipFree(n->d_unmasked);
     delete n;
     return hip_fail(e, "sb_net_create", __FILE__, __LINE__);
   }
