@@ -117,8 +117,10 @@ struct BufferWindow {
   using u4 = unsigned __attribute__((ext_vector_type(4)));
   using u2 = unsigned __attribute__((ext_vector_type(2)));
   // `at`: byte offset of the vector's first element (ignored parts: see `col`, `limit`); VEC moves the
-  // VW elements as one 16-byte access (all inside or all outside), otherwise element by element with
-  // elements at columns >= limit excluded.
+  // VW elements as one 16-byte access (all or none by `col`), otherwise element by element with elements
+  // at columns >= limit excluded.  A 16-byte access needs element alignment only, and the window's range
+  // check applies to each of its dwords on its own: the part inside the window is read or written, the
+  // rest reads zero / is dropped (measured on gfx950).
   template <bool VEC>
   __device__ __forceinline__ void load(T (&out)[Real<T>::VW], unsigned at, unsigned uniform, long col,
                                        long limit) const {
@@ -171,6 +173,13 @@ struct BufferWindow {
       for (int e = 0; e < VW; e++) v[e] = in[e];
       __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), rsrc,
                                              (int)(col < limit ? at : kOutside), (int)uniform, 0);
+    } else if (col + VW <= limit) {
+      // (rows that are no whole number of vectors: only the last vector of a row runs over its end, so
+      // in all but the last tile column this branch is taken by every lane)
+      typename Real<T>::vec_t v;
+#pragma unroll
+      for (int e = 0; e < VW; e++) v[e] = in[e];
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), rsrc, (int)at, (int)uniform, 0);
     } else {
 #pragma unroll
       for (int e = 0; e < VW; e++) {

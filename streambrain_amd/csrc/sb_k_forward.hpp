@@ -181,8 +181,12 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
 }
 
 // Main loop: x and W are read with 16-byte loads through bounds-checked buffer windows, so rows and
-// columns outside the matrices read zero and the loop body is loads + MFMAs only.  The last, partial K
-// chunk (and shapes without 16-byte alignment) take the guarded path.
+// columns outside the matrices read zero and the loop body is loads + MFMAs only.  Without VEC (shapes
+// without 16-byte alignment) the same loads start at any element -- multi-dword accesses need dword
+// alignment only -- and a vector that straddles the end of the tile also fetches a few columns of the
+// neighbouring tile, which land in accumulator columns the epilogue never reads (at the very end of W the
+// window's range check, which is per dword, returns zeros for them).  The last, partial K chunk takes the
+// guarded path.
 // One workgroup per CU is all the tiling provides at small batch sizes, so the register allocator is told
 // to aim for NWAVES/4 wavefronts per SIMD and spend the registers on loads in flight instead.
 //
@@ -278,7 +282,7 @@ void k_forward(ForwardArgs<T> a) {
   ForwardBias<T, NG, NWAVES>::load(bv, a.bias, j0, ncol);
   const long nfull = a.N / KC;  // chunks with all KC reduction indices inside the matrix
   SB_PHASE_MARK(0);
-  if (VEC) {
+  {
     // Chunk `w` first; every later chunk of this wavefront is NWAVES chunks further on.  x and W are
     // reached through bounds-checked buffer windows that start at the chunk (a scalar base address,
     // advanced with scalar instructions), so the per-lane offsets never change and the loop body is
@@ -347,12 +351,6 @@ void k_forward(ForwardArgs<T> a) {
     // partial last chunk (N % KC != 0): one wavefront takes it through the guarded path
     if (nfull * KC < a.N && w == (int)(nfull % NWAVES)) {
       load_guarded(nfull, xr[0], wr[0]);
-      compute(xr[0], wr[0]);
-    }
-  } else {
-    const long nchunks = (a.N + KC - 1) / KC;
-    for (long kc = w; kc < nchunks; kc += NWAVES) {
-      load_guarded(kc, xr[0], wr[0]);
       compute(xr[0], wr[0]);
     }
   }

@@ -116,6 +116,9 @@ __global__ __launch_bounds__(256) void k_trace_sums(TrainArgs<T> a) {
 // per CU; left alone the compiler takes 176 registers, which allows two).  Floats need no limit: 80-96.
 template <typename T>
 constexpr int train_waves_per_simd() { return sizeof(T) == 8 ? 4 : 1; }
+// VEC: Cij and W are stored as 16-byte vectors (M a multiple of VW), element by element otherwise.  Loads
+// are 16-byte accesses either way: one that runs over the end of a row of x, y or Cij fetches elements of
+// the next row into tile rows / columns outside the matrix, which are never stored or summed.
 // MB: mask bytes fetched per vector of VW columns -- 1 when Mc is a multiple of VW (every vector lies
 // inside one hypercolumn), VW otherwise.
 // PRE: Ci_next and Cj_next already hold the new traces (k_trace_sums): no column sums here.
@@ -198,8 +201,8 @@ void k_train_fused(TrainArgs<T> a) {
     const BufferWindow<T> xwin(a.x + b0 * a.N, (a.B - b0) * a.N), ywin(a.y + b0 * a.M, (a.B - b0) * a.M);
 #pragma unroll
     for (int m = 0; m < SP; m++) {
-      xwin.template load<VEC>(sx[m], xat[m], 0, i0 + VW * eg, a.N);
-      ywin.template load<VEC>(sy[m], yat[m], 0, ecol, a.M);
+      xwin.template load<true>(sx[m], xat[m], 0, i0 + VW * eg, a.N);
+      ywin.template load<true>(sy[m], yat[m], 0, ecol, a.M);
     }
   };
   request_chunk(0);
@@ -240,7 +243,7 @@ void k_train_fused(TrainArgs<T> a) {
   const unsigned pass_bytes = (unsigned)((long)RPP * a.M * ES);    // the next pass is RPP rows further on
   auto request_tile = [&]() {
 #pragma unroll
-    for (int k = 0; k < PASSES; k++) cwin.template load<VEC>(cpre[k], tat, k * pass_bytes, ecol, a.M);
+    for (int k = 0; k < PASSES; k++) cwin.template load<true>(cpre[k], tat, k * pass_bytes, ecol, a.M);
   };
 
   acc_t acc[2][2];
