@@ -84,7 +84,13 @@ int launch_forward_classify(hipStream_t st, T *act, const T *x, const T *W, cons
   const bool base_vec = (N % VW == 0) && (M % VW == 0) && aligned16(x) && aligned16(W);
   const long need = cdiv(Mc, GW);
   const long max_fused = sizeof(T) == 4 ? 4 : 7;
-  if (softmax && need <= max_fused) {
+  // The fused kernel runs one workgroup per hypercolumn and 16 batch rows, one workgroup per CU.  For wide
+  // hypercolumns (more than two column groups) whose tiles fill their last round of workgroups badly,
+  // tiles of two column groups plus a separate softmax pass are faster (1568 -> Hx200, batch 128, fused
+  // against separate: H = 16: 31.7 / 23.4 us, H = 30: 33.9 / 40.0, H = 48: 63.4 / 57.1, H = 64: 66.1 / 74.5).
+  const long fused_tiles = H * cdiv(B, 16), cus_ = device_cu_count();
+  const bool enough_tiles = need <= 2 || 20 * fused_tiles >= 17 * cdiv(fused_tiles, cus_) * cus_;
+  if (softmax && need <= max_fused && enough_tiles) {
     const bool vec = base_vec && (Mc % VW == 0);
     a.col_tiles = H;
     // Hypercolumns that need 7 column blocks of 16 (97..112 columns, e.g. 100): the last group runs
