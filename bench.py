@@ -2,7 +2,7 @@
 """Benchmark of the BCPNN layer training step on one MI355X.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
-  python bench.py --workload dense|wide64|stl10|largest     (other configurations, see LARGE below)
+  python bench.py --workload dense|mnist15x200|wide64|stl10|largest    (other configurations, see LARGE below)
 
 Workload: the MNIST-shaped 2-layer network, float32, batch 128, 60000 seeded
 synthetic samples; input 784 pixels complementary-coded to 1568 units (~19% nonzero pixels, uniform
@@ -201,6 +201,9 @@ LARGE = {
                   what="configs[3]: STL-10-shaped layer 55296 -> 200x100, float32, batch 256, mask density 0.05"),
     "largest": dict(n=65536, h=1000, mc=100, batch=1024, density=1.0, dtype=np.float32, samples=4096, nonzero=0.2,
                     what="configs[4]: 65536 -> 1000x100, float32, batch 1024, binary inputs, dense mask"),
+    "mnist15x200": dict(n=1568, h=15, mc=200, batch=128, density=0.1, dtype=np.float32, samples=60000, nonzero=0.19,
+                        what="the reference example script's own MNIST layer: 1568 -> 15x200, float32, batch 128, "
+                             "mask density 0.1"),
     "wide64": dict(n=1568, h=100, mc=100, batch=512, density=0.1, dtype=np.float64, samples=60000, nonzero=0.19,
                    what="configs[2]: 1568 -> 100x100, float64, batch 512, mask density 0.1"),
 }
