@@ -362,8 +362,39 @@ def test_argmax_rows(k, oracle, dtype):
 @pytest.mark.parametrize("B,N,H,Mc,h", [(16, 40, 3, 8, None), (16, 40, 3, 8, 1), (128, 1568, 30, 100, None),
                                         (128, 1568, 30, 100, 7), (96, 300, 4, 25, 3), (9, 33, 2, 7, 0)])
 def test_plastic_train_step(k, oracle, dtype, B, N, H, Mc, h):
+    _check_plastic_train_step(k, oracle, dtype, B, N, H, Mc, h, np.random.default_rng(B + N + H + Mc))
+
+
+def _random_shapes(seed, count):
+    """Shapes off every tiling's grid: mostly odd widths, batches around the 16- and 32-row boundaries."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        B = int(rng.choice([1, 2, 15, 16, 17, 31, 33, 47, 64, 100, 129]))
+        N = int(rng.integers(1, 400))
+        H = int(rng.integers(1, 7))
+        Mc = int(rng.choice([1, 2, 3, 5, 9, 16, 17, 31, 33, 50, 63, 65, 100, 101, 127, 130]))
+        out.append((B, N, H, Mc))
+    return out
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("B,N,H,Mc", _random_shapes(2024, 24))
+def test_random_shapes_forward_and_train_step(k, oracle, dtype, B, N, H, Mc):
+    rng = np.random.default_rng(B + 3 * N + 5 * H + 7 * Mc)
+    M = H * Mc
+    x = rng.random((B, N)).astype(dtype)
+    W = (0.1 * rng.standard_normal((N, M))).astype(dtype)
+    b = (0.1 * rng.random(M)).astype(dtype)
+    ref = oracle.softmax_minicolumns(oracle.update_state(np.zeros((B, M), dtype=dtype), W, b, x), H, Mc)
+    scale = max(1.0, np.sqrt(N / 64.0)) if dtype == np.float32 else 4.0
+    assert_close(k.compute_activation(W, b, x, H, Mc), ref, dtype, "forward", scale)
+    h = int(rng.integers(0, H)) if rng.random() < 0.5 else None
+    _check_plastic_train_step(k, oracle, dtype, B, N, H, Mc, h, rng, must_rewire=False)
+
+
+def _check_plastic_train_step(k, oracle, dtype, B, N, H, Mc, h, rng, must_rewire=True):
     import scipy.special
-    rng = np.random.default_rng(B + N + H + Mc)
     M = H * Mc
     tau, khalf, pmin, taubdt = 0.006908854922437549, -139.02586632856327, 0.06195283356566607, \
         0.02218100432360414
@@ -387,7 +418,7 @@ def test_plastic_train_step(k, oracle, dtype, B, N, H, Mc, h):
         oracle.update_mask(r["wmask"], r["weights"], r["Ci"], r["Cj"], r["Cij"], cthr, H, Mc, h, 16)
     oracle.apply_mask(r["weights"], r["wmask"], H, Mc)
     assert np.array_equal(got["wmask"], r["wmask"])
-    if h is not None and N > 100:
+    if must_rewire and h is not None and N > 100:
         assert not np.array_equal(r["wmask"], st["wmask"]), "the case is meant to rewire"
     assert np.array_equal(got["Ci"], r["Ci"]) and np.array_equal(got["Cj"], r["Cj"])
     assert np.array_equal(got["kbi"], r["kbi"])
