@@ -336,6 +336,8 @@ def main():
     ap.add_argument("--steps", type=int, default=938)
     ap.add_argument("--warmup", type=int, default=60)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-baseline-seconds", type=float, default=15.0,
+                    help="length of the CPU baseline's sample")
     ap.add_argument("--samples", type=int, default=N_SAMPLES)
     ap.add_argument("--workload", choices=["mnist"] + sorted(LARGE), default="mnist",
                     help="mnist (default): the headline configuration; the others: one layer of a larger "
@@ -438,7 +440,7 @@ def main():
         },
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(x, y)
+        result["cpu_baseline"] = cpu_baseline(x, y, budget_s=args.cpu_baseline_seconds)
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))

@@ -1,0 +1,47 @@
+"""bench.py on the GPU: a short run prints exactly one JSON line with the fields the measurement contract
+names, and its figures are consistent with each other."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _run(*args):
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), *args], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [ln for ln in r.stdout.splitlines() if ln.strip()]
+    assert len(lines) == 1, lines
+    return json.loads(lines[0])
+
+
+def test_headline_line_short_run():
+    b = _run("--steps", "60", "--warmup", "10", "--samples", "8960", "--cpu-baseline-seconds", "2")
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in b, key
+    assert b["n_gpus"] == 1 and b["steps"] == 60 and b["warmup"] == 10 and b["higher_is_better"] is True
+    assert b["unit"] == "samples/s" and b["dtype"] == "f32" and b["vs_baseline"] is None
+    assert "workload" in b["config"] and "model" not in b["config"]
+    # value = samples / time; 60 full batches of 128 in the timed region
+    assert b["value"] == pytest.approx(60 * 128 / (b["ms_per_step"] * 60 / 1e3), rel=1e-6)
+    r = b["roofline"]
+    assert r["bound"] == "hbm" and r["unit"] == "GB/s" and r["peak"] == 8000.0
+    assert r["frac"] == pytest.approx(r["achieved"] / r["peak"], rel=1e-9) and 0.0 < r["frac"] < 1.0
+    assert r["achieved"] == pytest.approx(r["algorithmic_bytes_per_launch"] / (r["avg_launch_us"] * 1e-6) / 1e9, rel=1e-6)
+    c = b["cpu_baseline"]
+    assert c["kind"] == "port" and c["cores"] >= 1 and c["value"] > 0 and c["unit"] == "samples/s"
+    assert b["value"] > c["value"]
+
+
+def test_other_workload_line():
+    b = _run("--workload", "dense", "--steps", "40", "--warmup", "10")
+    assert b["n_gpus"] == 1 and b["dtype"] == "f32" and b["cpu_baseline"] is None
+    assert b["roofline"]["bound"] in ("hbm", "mfma") and 0.0 < b["roofline"]["frac"] < 1.0
+    assert "configs[0]" in b["config"]["workload"]
