@@ -50,14 +50,16 @@ constexpr int forward_rows_waves_per_simd() {
 // RB: row blocks per workgroup, as in k_forward: 16*RB batch rows share every gathered W vector.
 // XT: x is read from the blocked copy `xt` instead of a.x: the 16 lanes p of an entry then read 16
 // consecutive elements (one 64-byte access) instead of one element each of 16 rows.
-template <typename T, int NG, int NWAVES, int RB = 1, bool XT = false>
+// LW: column blocks of the last group, as in k_forward (a hypercolumn of 100 columns takes 7 blocks of
+// 16 instead of 8: the last group's lanes load LW consecutive columns).
+template <typename T, int NG, int NWAVES, int RB = 1, bool XT = false, int LW = Real<T>::VW>
 __global__ __launch_bounds__(64 * NWAVES)
 __attribute__((amdgpu_waves_per_eu(forward_rows_waves_per_simd<T, NG, RB>(),
                                    forward_rows_waves_per_simd<T, NG, RB>())))
 void k_forward_rows(ForwardRowsArgs<T> ar) {
   const ForwardArgs<T> &a = ar.f;
   constexpr int VW = Real<T>::VW;
-  using TC = TileCols<T, NG, VW>;
+  using TC = TileCols<T, NG, LW>;
   constexpr int KC = 4 * VW;      // list entries per chunk
   constexpr int SEG = 2048;       // list entries per segment
   constexpr int SEGC = SEG / KC;  // chunks per segment
@@ -148,9 +150,15 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
       const long roff = (long)(r < 0 ? 0 : r) * a.M;
 #pragma unroll
       for (int g = 0; g < NG; g++) {
-        const vec_t v = *reinterpret_cast<const vec_t *>(wcol[g] + roff);
+        if (TC::gwidth(g) == VW) {
+          const vec_t v = *reinterpret_cast<const vec_t *>(wcol[g] + roff);
 #pragma unroll
-        for (int c2 = 0; c2 < VW; c2++) wo[s][g][c2] = v[c2];
+          for (int c2 = 0; c2 < VW; c2++) wo[s][g][c2] = v[c2];
+        } else {
+          const PackedCols<T, LW> v = *reinterpret_cast<const PackedCols<T, LW> *>(wcol[g] + roff);
+#pragma unroll
+          for (int c2 = 0; c2 < LW; c2++) wo[s][g][c2] = v.v[c2];
+        }
       }
     }
   };
@@ -161,8 +169,10 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
       for (int g = 0; g < NG; g++)
 #pragma unroll
         for (int c = 0; c < VW; c++)
+          if (c < TC::gwidth(g)) {
 #pragma unroll
-          for (int r = 0; r < RB; r++) acc[r][g][c] = Real<T>::mfma(xi[r][s], wi[s][g][c], acc[r][g][c]);
+            for (int r = 0; r < RB; r++) acc[r][g][c] = Real<T>::mfma(xi[r][s], wi[s][g][c], acc[r][g][c]);
+          }
   };
 
   for (long seg0 = 0;;) {
@@ -203,7 +213,7 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
 #pragma unroll
   for (int r = 0; r < RB; r++) {
     if (r > 0) __syncthreads();  // the previous row block's sums have been read
-    forward_finish<T, NG, true, NWAVES, VW>(acc[r], bv, red, a.act, a.B, a.M, b0 + 16 * r, j0, ncol);
+    forward_finish<T, NG, true, NWAVES, LW>(acc[r], bv, red, a.act, a.B, a.M, b0 + 16 * r, j0, ncol);
   }
   SB_PHASE_MARK(3);
 }

@@ -147,7 +147,7 @@ bool forward_rows_supported(const T *W, long N, long H, long Mc) {
          cdiv(Mc, 16 * VW) <= (sizeof(T) == 4 ? 4 : 7) && 16 * N * (long)sizeof(T) < (1L << 31);
 }
 
-template <typename T, int NG>
+template <typename T, int NG, int LW = Real<T>::VW>
 static int forward_rows_variant(hipStream_t st, ForwardRowsArgs<T> a) {
   ProfScope prof_(st, K_FORWARD);
   // four wavefronts measured best (8: 8.8 us, 4: 8.2 us, 2: 9.9 us, 16: 10.7 us at 1568 -> 30x100, density 0.1)
@@ -169,22 +169,22 @@ static int forward_rows_variant(hipStream_t st, ForwardRowsArgs<T> a) {
   const dim3 g((unsigned)grid), blk(64 * NW);
   if (a.xt) {  // the batch is also at hand in blocks of 16 rows
     if constexpr (fits4) {
-      if (rb == 4) hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 4, true>), g, blk, 0, st, a);
+      if (rb == 4) hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 4, true, LW>), g, blk, 0, st, a);
     }
     if (rb == 4) {
     } else if (rb == 2)
-      hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 2, true>), g, blk, 0, st, a);
+      hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 2, true, LW>), g, blk, 0, st, a);
     else
-      hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 1, true>), g, blk, 0, st, a);
+      hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 1, true, LW>), g, blk, 0, st, a);
   } else {
     if constexpr (fits4) {
-      if (rb == 4) hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 4>), g, blk, 0, st, a);
+      if (rb == 4) hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 4, false, LW>), g, blk, 0, st, a);
     }
     if (rb == 4) {
     } else if (rb == 2)
-      hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 2>), g, blk, 0, st, a);
+      hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 2, false, LW>), g, blk, 0, st, a);
     else
-      hipLaunchKernelGGL((k_forward_rows<T, NG, NW>), g, blk, 0, st, a);
+      hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 1, false, LW>), g, blk, 0, st, a);
   }
   SB_LAUNCH_CHECK();
   return 0;
@@ -200,6 +200,12 @@ int launch_forward_rows(hipStream_t st, T *act, const T *x, const T *W, const T 
   SB_REQUIRE(forward_rows_supported<T>(W, N, H, Mc), "shape not supported by the row-list forward kernel");
   ForwardRowsArgs<T> a{{act, x, W, bias, B, N, H * Mc, Mc, H, cdiv(B, 16)}, rows, row_cnt, cap, x_blocked};
   const long need = cdiv(Mc, 16 * Real<T>::VW);
+  // hypercolumns of 7 column blocks of 16 (97..112 columns): the last group runs with 3 (float) or 1
+  // (double) blocks, provided none of its vectors straddles the end of the hypercolumn (as in launch_forward)
+  {
+    constexpr int VW = Real<T>::VW, GW = 16 * VW, NGL = 8 / VW, LWL = 7 - (NGL - 1) * VW;
+    if (cdiv(Mc, 16) == 7 && (Mc - (NGL - 1) * GW) % LWL == 0) return forward_rows_variant<T, NGL, LWL>(st, a);
+  }
   if (need <= 1) return forward_rows_variant<T, 1>(st, a);
   if (need <= 2) return forward_rows_variant<T, 2>(st, a);
   if (need <= 4) return forward_rows_variant<T, 4>(st, a);
