@@ -84,40 +84,72 @@ __global__ __launch_bounds__(256) void k_forward_skinny(T *act, const T *x, cons
 }
 
 // The fused training pass of k_train_fused (same arguments, same results within rounding) for M <= 32:
-// one workgroup per R rows of Cij; thread (r, j) walks the batch once, accumulating its x^T y element
-// and, in batch order and without FMA contraction, the column sums its row's Ci and its column's Cj
-// are made of -- the reference's order, so the traces are bit-exact as in the tiled kernel.
+// one workgroup per R rows of Cij (skinny_train_rows), thread (r, j) owning one element.  The workgroup stages its
+// R columns of x and all of y in LDS, `bc` batch rows at a time, with every load of a chunk in flight at
+// once (a row of x contributes R consecutive elements, a row of y all M); each thread then walks the
+// chunk in LDS, accumulating its x^T y element and, in batch order and without FMA contraction, the
+// column sums its row's Ci and its column's Cj are made of -- the reference's order, so the traces are
+// bit-exact as in the tiled kernel.  Rows past the batch are staged as zeros, which change no sum.
+// bc (set by the launcher): at most kSkinnyLoads passes of either staging loop, at most kSkinnyStage
+// staged elements, byte offsets of a chunk of x below 2 GiB.
+// Rows of Cij per workgroup: as many as fit 256 threads, at most 32 (with fewer columns than 8 some threads
+// only stage; more rows would shorten the chunks the staging loops can cover).
+__host__ __device__ constexpr int skinny_train_rows(long M) { return 256 / M < 32 ? (int)(256 / M) : 32; }
+constexpr int kSkinnyLoads = 16;
+constexpr int kSkinnyStage = 8192;
 template <typename T>
-__global__ __launch_bounds__(256) void k_train_skinny(TrainArgs<T> a) {
+__global__ __launch_bounds__(256) void k_train_skinny(TrainArgs<T> a, int bc) {
   using Rl = Real<T>;
+  __shared__ T stage[kSkinnyStage];
   const int tid = threadIdx.x;
   const int M = (int)a.M;
-  const int R = 256 / M;
+  const int R = skinny_train_rows(M);
   const int j = tid % M, r = tid / M;
-  const long i = (long)blockIdx.x * R + r;
-  if (r >= R || i >= a.N) return;  // no barriers below
+  const long i0 = (long)blockIdx.x * R, i = i0 + r;
+  const bool mine = r < R && i < a.N;  // this thread owns an element of Cij
+  T *xs = stage, *ys = stage + bc * R;
+  // staging roles: x by (row xb of a pass, column xr), y by (row yb, column yj)
+  const int xrows = 256 / R, xb = tid / R, xr = tid % R;  // xrows * R <= 256 threads load x
+  const int yrows = 256 / M, yb = tid / M, yj = tid % M;
+  const bool xload = xb < xrows && i0 + xr < a.N, yload = yb < yrows;
+  constexpr unsigned ES = sizeof(T);
+  const T cij_old = mine ? a.Cij[i * a.M + j] : T(0);  // requested first, used last
   T dot = T(0), sx = T(0), sy = T(0);
-  const T *xp = a.x + i, *yp = a.y + j;
-  // 32 batch rows of loads in flight (branch-free: past the batch the last row is re-read and counts
-  // as 0), then the ordered arithmetic; the pointers advance by one row per load
-  for (long b0 = 0; b0 < a.B; b0 += 32) {
-    T xv[32], yv[32];
+  for (long b0 = 0; b0 < a.B; b0 += bc) {
+    const long left = a.B - b0;  // rows of this chunk inside the batch: min(left, bc)
+    const BufferWindow<T> xwin(a.x + b0 * a.N + i0, (left - 1) * a.N + (a.N - i0)),
+        ywin(a.y + b0 * a.M, left * a.M);
+    T xv[kSkinnyLoads], yv[kSkinnyLoads];
 #pragma unroll
-    for (int k = 0; k < 32; k++) {
-      const bool live = b0 + k < a.B;  // uniform; the pointers stop at the last row of the batch
-      xv[k] = *xp, yv[k] = *yp;
-      xp += live && b0 + k + 1 < a.B ? a.N : 0;
-      yp += live && b0 + k + 1 < a.B ? a.M : 0;
+    for (int k = 0; k < kSkinnyLoads; k++) {
+      const int bx = xb + k * xrows, by = yb + k * yrows;
+      T one[1];
+      xwin.template load_n<1>(one, xload && bx < bc ? (unsigned)(((long)bx * a.N + xr) * ES)
+                                                    : BufferWindow<T>::kOutside);
+      xv[k] = one[0];
+      ywin.template load_n<1>(one, yload && by < bc ? (unsigned)(((long)by * a.M + yj) * ES)
+                                                    : BufferWindow<T>::kOutside);
+      yv[k] = one[0];
     }
+    if (b0 > 0) __syncthreads();  // the previous chunk has been consumed
 #pragma unroll
-    for (int k = 0; k < 32; k++) {
-      const bool live = b0 + k < a.B;
-      const T xk = live ? xv[k] : T(0), yk = live ? yv[k] : T(0);
-      dot += xk * yk;
-      sx = Rl::add(sx, xk);
-      sy = Rl::add(sy, yk);
+    for (int k = 0; k < kSkinnyLoads; k++) {
+      const int bx = xb + k * xrows, by = yb + k * yrows;
+      if (xb < xrows && bx < bc) xs[bx * R + xr] = xv[k];
+      if (yload && by < bc) ys[by * M + yj] = yv[k];
+    }
+    __syncthreads();
+    if (mine) {
+      const int rows = left < bc ? (int)left : bc;
+      for (int b = 0; b < rows; b++) {
+        const T xk = xs[b * R + r], yk = ys[b * M + j];
+        dot += xk * yk;
+        sx = Rl::add(sx, xk);
+        sy = Rl::add(sy, yk);
+      }
     }
   }
+  if (!mine) return;
   const T ci = trace_next<T>(a.Ci[i], sx, a), cj = trace_next<T>(a.Cj[j], sy, a);
   if (j == 0) a.Ci_next[i] = ci;
   if (i == 0) {
@@ -128,7 +160,7 @@ __global__ __launch_bounds__(256) void k_train_skinny(TrainArgs<T> a) {
       a.kbi[j] = kb;
     }
   }
-  T cn = a.Cij[i * a.M + j] * a.omt + dot * (a.invB * a.tau);
+  T cn = cij_old * a.omt + dot * (a.invB * a.tau);
   cn = fmax(cn, T(0));
   a.Cij[i * a.M + j] = cn;
   const T wgt = weight_from_traces<T>(cn, trace_reciprocal<T>(ci, a.cthr), trace_reciprocal<T>(cj, a.cthr),

@@ -253,10 +253,16 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   a.panel_cols = B * N * (long)sizeof(T) > (2L << 20) ? 8u : 1u;
   a.by_panel = FastDiv::of(a.tiles_i * a.panel_cols); a.by_Mc = FastDiv::of(Mc);
   if (M <= 32) {  // a handful of output units: plain vector arithmetic
-    const long rows = 256 / M;
+    const long rows = skinny_train_rows(M);
     SB_REQUIRE(cdiv(N, rows) < (1L << 31), "too many rows for one launch");
     ProfScope prof_(st, K_TRAIN_FUSED);
-    hipLaunchKernelGGL((k_train_skinny<T>), dim3((unsigned)cdiv(N, rows)), dim3(256), 0, st, a);
+    // batch rows staged per chunk (see the kernel)
+    long bc = kSkinnyLoads * (256 / rows) < kSkinnyLoads * (256 / M) ? kSkinnyLoads * (256 / rows) : kSkinnyLoads * (256 / M);
+    if (bc > kSkinnyStage / (rows + M)) bc = kSkinnyStage / (rows + M);
+    if (bc > ((1L << 31) - 1) / (N * (long)sizeof(T))) bc = ((1L << 31) - 1) / (N * (long)sizeof(T));
+    if (bc > B) bc = B;
+    SB_REQUIRE(bc >= 1, "layer too wide for the small-output training kernel");
+    hipLaunchKernelGGL((k_train_skinny<T>), dim3((unsigned)cdiv(N, rows)), dim3(256), 0, st, a, (int)bc);
     SB_LAUNCH_CHECK();
     return 0;
   }
