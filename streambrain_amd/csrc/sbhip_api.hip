@@ -176,6 +176,10 @@ struct sb_net {
   int64_t *d_perm = nullptr;
   int64_t *h_perm = nullptr;  // pinned staging
   hipEvent_t perm_copied = nullptr;
+  // While only the last layer trains, the layers below it are frozen: their output for every training
+  // sample is computed once (Hc, data-set order) and shuffled per epoch like the images (Hcp).
+  void *Hc = nullptr, *Hcp = nullptr;
+  int Hc_layer = -1;  // Hc holds the activations of this layer for the current training set (-1: none)
   unsigned long long *d_correct = nullptr;   // evaluate's counter
   unsigned long long *d_unmasked = nullptr;  // layer_check_masked's counter
 };
@@ -345,6 +349,43 @@ static int layer_mask_replaced(Layer &L, const uint8_t *mask) {
   return launch_mask_rows(g_ctx.stream, L.rows, L.row_cnt, L.wmask, L.N, L.H, L.rows_cap, 0, L.H);
 }
 
+// Largest cache of frozen activations kept (bytes, both copies together); beyond it they are recomputed.
+static const size_t kFrozenCacheLimit = (size_t)16 << 30;
+
+static int drop_frozen_cache(sb_net *net) {
+  if (!net->Hc && !net->Hcp) {
+    net->Hc_layer = -1;
+    return 0;
+  }
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  int rc = free_dev(net->Hc) | free_dev(net->Hcp);
+  net->Hc_layer = -1;
+  return rc;
+}
+
+// Activations of layer `upto` for all training samples in data-set order, in batches of maxB (the batch
+// size the training steps use, so the same kernel variants run).
+template <typename T>
+static int build_frozen_cache(sb_net *net, int upto, long maxB) {
+  const long Ns = net->Ns, Mo = net->layers[upto].M;
+  int rc = drop_frozen_cache(net);
+  if (rc) return rc;
+  SB_HIP(hipMalloc(&net->Hc, (size_t)Ns * Mo * sizeof(T)));
+  SB_HIP(hipMalloc(&net->Hcp, (size_t)Ns * Mo * sizeof(T)));
+  for (long lo = 0; lo < Ns; lo += maxB) {
+    const long B = lo + maxB <= Ns ? maxB : Ns - lo;
+    const T *x = (const T *)net->X + lo * net->NF;
+    for (int l = 0; l <= upto; l++) {
+      if ((rc = layer_forward<T>(net, net->layers[l], x, B))) return rc;
+      x = (const T *)net->layers[l].act;
+    }
+    SB_HIP(hipMemcpyAsync((T *)net->Hc + lo * Mo, x, (size_t)B * Mo * sizeof(T), hipMemcpyDeviceToDevice,
+                          g_ctx.stream));
+  }
+  net->Hc_layer = upto;
+  return 0;
+}
+
 template <typename T>
 static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h_sample_perm,
                              const int64_t *h_hc_perm, long epoch, long first_batch, long n_batches,
@@ -365,6 +406,10 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
   if (rc) return rc;
   const bool permute = first_batch == 0;  // a later range continues the epoch already laid out
   SB_REQUIRE(permute || net->Xp, "the epoch's first batches have not been run");
+  // a training step of a layer below the last changes what the cache was computed from
+  if (!last && (rc = drop_frozen_cache(net))) return rc;
+  const long Mprev = layer > 0 ? net->layers[layer - 1].M : 0;
+  const bool cache_fits = last && layer > 0 && 2 * (size_t)Ns * Mprev * sizeof(T) <= kFrozenCacheLimit;
   if (permute) {
     SB_REQUIRE(h_sample_perm, "sample order missing");
     for (long r = 0; r < Ns; r++)
@@ -395,7 +440,14 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
     if (last)
       if ((rc = launch_gather_rows<T>(st, (T *)net->Yp, (const T *)net->Y, net->d_perm, Ns, net->NC)))
         return rc;
+    if (cache_fits) {
+      if (net->Hc_layer != layer - 1 && (rc = build_frozen_cache<T>(net, layer - 1, maxB))) return rc;
+      if ((rc = launch_gather_rows<T>(st, (T *)net->Hcp, (const T *)net->Hc, net->d_perm, Ns, Mprev))) return rc;
+    } else if (last && (rc = drop_frozen_cache(net))) {
+      return rc;
+    }
   }
+  const bool cached = cache_fits && net->Hc_layer == layer - 1;
 
   const long period = nb / (target.H + 1);  // _cpu_base_backend.py:297-299
   for (long i = first_batch; i < first_batch + n_batches; i++) {
@@ -403,9 +455,13 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
     const long B = (lo + maxB <= Ns) ? maxB : Ns - lo;
     const T *x = (const T *)net->Xp + lo * net->NF;
     const T *xb = net->XpB_batch == maxB ? (const T *)net->XpB + lo * net->NF : nullptr;  // lo % 16 == 0
-    for (int l = 0; l < layer; l++) {
-      if ((rc = layer_forward<T>(net, net->layers[l], x, B, l == 0 ? xb : nullptr))) return rc;
-      x = (const T *)net->layers[l].act;
+    if (cached) {
+      x = (const T *)net->Hcp + lo * Mprev;
+    } else {
+      for (int l = 0; l < layer; l++) {
+        if ((rc = layer_forward<T>(net, net->layers[l], x, B, l == 0 ? xb : nullptr))) return rc;
+        x = (const T *)net->layers[l].act;
+      }
     }
     long h = -1;
     if (!last && epoch > 0 && period > 0 && i % period == 0) {
@@ -764,6 +820,8 @@ int sb_net_training_done(sb_net *net) {
   rc |= free_dev(net->X); rc |= free_dev(net->Y); rc |= free_dev(net->Xp); rc |= free_dev(net->Yp);
   rc |= free_dev(net->XpB);
   net->XpB_batch = 0;
+  rc |= free_dev(net->Hc); rc |= free_dev(net->Hcp);
+  net->Hc_layer = -1;
   rc |= free_dev(p);
   net->d_perm = nullptr;
   if (net->h_perm) SB_HIP(hipHostFree(net->h_perm));
@@ -826,6 +884,7 @@ int sb_net_set_layer_state(sb_net *net, int layer, const char *name, const void 
   SB_REQUIRE(bytes == s.bytes, "size mismatch");
   rc = sb_memcpy_h2d(s.ptr, h_src, bytes);
   if (rc) return rc;
+  if ((rc = drop_frozen_cache(net))) return rc;  // (whatever layer: the cache is cheap to rebuild)
   Layer &L = net->layers[layer];
   if (s.ptr == L.W) L.w_masked = false, L.w_unchecked = true;
   if (s.ptr == L.wmask)

@@ -111,6 +111,35 @@ def test_odd_shaped_networks_f64(hb, n_pix, H, Mc, n_out, Ns, B, density):
     assert rel_err(g.forward(Xt, 7), r.forward(Xt.astype(np.float64))) <= 1e-10
 
 
+def test_classifier_epochs_follow_changes_below_them_f64(hb):
+    """While only the output layer trains, the backend keeps the hidden layer's activations of the training
+    set instead of recomputing them every epoch.  Whatever changes the hidden layer in between -- its own
+    training, state written from outside -- must show in the next classifier epoch as it does in the
+    cpu-backend restatement, which recomputes everything."""
+    from oracle import cpu_backend as ob
+    rng = np.random.default_rng(77)
+    n_pix, H, Mc, n_out, Ns, B = 30, 4, 12, 5, 150, 16
+    X, Y = synthetic_images(rng, Ns, n_pix), one_hot_labels(rng, Ns, n_out)
+    Xt = synthetic_images(rng, 40, n_pix)
+    nets = []
+    for backend in (hb, ob):
+        net = build_two_layer(backend, 2 * n_pix, H, Mc, n_out, dict(MNIST_HP, l1_density=0.4), np.float64, seed=3)
+        net.fit(X, Y, B, [(0, 2)])
+        net.fit(X, Y, B, [(1, 2)])            # activations kept over these two epochs
+        net.fit(X, Y, B, [(0, 1)])            # the hidden layer moves on
+        net.fit(X, Y, B, [(1, 1)])
+        w = np.array(net._layers[0].weights)  # state written from outside
+        w[::3] *= 0.5
+        net._layers[0].weights = w
+        net.fit(X, Y, B, [(1, 2)])
+        net.fit(X[:100], Y[:100], B, [(1, 1)])  # another training set
+        nets.append(net)
+    g, r = nets
+    assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
+    _compare_states(g, r, 1e-10)
+    assert np.array_equal(g.predict(Xt, B), r.predict(Xt, B))
+
+
 def test_small_network_one_epoch_f32(hb):
     # float32, one epoch per layer (13 batches, short last one).  Stated drift bound after one epoch:
     # 1e-4 relative (rounding differences of ~1e-7 per step, amplified by the log of small traces).
