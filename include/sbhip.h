@@ -212,6 +212,9 @@ int sb_net_training_done(sb_net *net);
  *                             (:297-302), used when epoch_index > 0; may be NULL for the last layer;
  * the last layer trains on the labels, any other on its own activation; ends with train_finalize.
  * When n_batches / (H + 1) is zero the reference divides by zero; here no rewiring happens.
+ * While the last layer trains, the layers below it do not change: their activations of the training set
+ * are computed in its first epoch and kept (two copies of [n_samples, its input width], as long as
+ * they stay below 16 GiB) until a lower layer trains, state is written or the training set is replaced.
  * Asynchronous: returns once the epoch is enqueued. */
 int sb_net_train_epoch(sb_net *net, int layer, long maximal_batch_size,
                        const int64_t *h_sample_perm, const int64_t *h_hc_perm, long epoch_index);
