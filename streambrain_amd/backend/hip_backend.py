@@ -154,33 +154,35 @@ class Network:
         self._layers.append(layer)
 
     def fit(self, training_data, training_labels, maximal_batch_size, schedule):
-        training_data = np.ascontiguousarray(training_data.astype(self.dtype))
-        training_labels = np.ascontiguousarray(training_labels.astype(self.dtype))
+        # (converted only when needed: the backend object copies the arrays to the device anyway)
+        training_data = np.ascontiguousarray(training_data, dtype=self.dtype)
+        training_labels = np.ascontiguousarray(training_labels, dtype=self.dtype)
         self.net.initiate_training(training_data, training_labels)
         n_samples = training_data.shape[0]
         for layer, epochs in schedule:
             for epoch in range(epochs):
                 print('Layer - %d/%d' % (layer + 1, len(self._layers)), flush=True)
-                # the two draws of an epoch, in the reference's order
-                idx = np.random.permutation(range(n_samples))
-                hypercolumns_shuffled = np.random.permutation(range(self._layers[layer].hypercolumns))
+                # the two draws of an epoch, in the reference's order (permutation(n) draws and returns what
+                # the reference's permutation(range(n)) does, without building the range element by element)
+                idx = np.random.permutation(n_samples)
+                hypercolumns_shuffled = np.random.permutation(self._layers[layer].hypercolumns)
                 self.net.train_epoch(layer, maximal_batch_size, idx.astype(np.int64),
                                      hypercolumns_shuffled.astype(np.int64), epoch)
         self.net.synchronize()
         self.net.training_done()
 
     def evaluate(self, images, labels, maximal_batch_size):
-        images = np.ascontiguousarray(images.astype(self.dtype))
-        labels = np.ascontiguousarray(labels.astype(self.dtype))
+        images = np.ascontiguousarray(images, dtype=self.dtype)
+        labels = np.ascontiguousarray(labels, dtype=self.dtype)
         correct, total = self.net.evaluate_counts(images, labels, maximal_batch_size)
         return np.array([correct]), np.array([total])
 
     def predict(self, images, maximal_batch_size):
-        images = np.ascontiguousarray(images.astype(self.dtype))
+        images = np.ascontiguousarray(images, dtype=self.dtype)
         return self.net.predict(images, maximal_batch_size)
 
     def forward(self, images, maximal_batch_size=None, last_layer=None):
-        images = np.ascontiguousarray(images.astype(self.dtype))
+        images = np.ascontiguousarray(images, dtype=self.dtype)
         if last_layer is None:
             last_layer = len(self._layers) - 1
         return self.net.forward(images, last_layer, maximal_batch_size or max(1, images.shape[0]))
