@@ -208,6 +208,9 @@ int launch_forward_rows(hipStream_t st, T *act, const T *x, const T *W, const T 
   {
     constexpr int VW = Real<T>::VW, GW = 16 * VW, NGL = 8 / VW, LWL = 7 - (NGL - 1) * VW;
     if (cdiv(Mc, 16) == 7 && (Mc - (NGL - 1) * GW) % LWL == 0) return forward_rows_variant<T, NGL, LWL>(st, a);
+    // and of 13 column blocks (193..208 columns, 200 among them): one block in the last group
+    constexpr int NGM = 16 / VW - (VW == 2 ? 1 : 0);  // float: 4 groups (12 + 1 blocks); double: 7 (12 + 1)
+    if (cdiv(Mc, 16) == 13) return forward_rows_variant<T, NGM, 1>(st, a);
   }
   if (need <= 1) return forward_rows_variant<T, 1>(st, a);
   if (need <= 2) return forward_rows_variant<T, 2>(st, a);
