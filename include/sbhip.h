@@ -127,6 +127,21 @@ int sb_update_weights_f64(double *d_Ci, double *d_Cj, double *d_Cij, const doubl
                           const double *d_a_o, double taupdt, double *d_W, double cthr, long B,
                           long N, long M);
 
+/* sb_update_weights_f32 for callers that cannot call hipMalloc (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid allocation).  No counterpart in the reference.  Same arguments
+ * and results as sb_update_weights_f32; the intermediate new Ci / Cj live in a static device array of
+ * SB_NOALLOC_MAX_UNITS floats (1 MiB, held by every GPU the library runs on until the process ends)
+ * instead of a buffer the library grows on demand, so the call allocates and frees nothing.  Returns
+ * SB_ERR_UNSUPPORTED when N + M > SB_NOALLOC_MAX_UNITS, SB_ERR_STATE between sb_profile_start and
+ * sb_profile_stop (event brackets allocate).  Every call of a process on a GPU shares the one array,
+ * which keeps the last call's contents (the kernel overwrites what it reads back, nothing needs
+ * clearing): two calls that overlapped on a GPU would race.  The library's single stream orders them;
+ * as with every entry point, do not call from two threads at once. */
+#define SB_NOALLOC_MAX_UNITS 262144
+int sb_update_weights_noalloc_f32(float *d_Ci, float *d_Cj, float *d_Cij, const float *d_a_i,
+                                  const float *d_a_o, float taupdt, float *d_W, float cthr, long B,
+                                  long N, long M);
+
 /* replaces update_bias_float32/64, kernels_openmp_internal.cc:207-220,386-396 */
 int sb_update_bias_f32(float *d_bias, const float *d_Cj, float cthr, long M);
 int sb_update_bias_f64(double *d_bias, const double *d_Cj, double cthr, long M);

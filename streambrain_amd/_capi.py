@@ -48,6 +48,7 @@ _PLAIN_SIGS = {
     "sb_memcpy_d2d": [_P, _P, _Z],
     "sb_fill_bytes": [_P, _I, _Z],
     "sb_mask_rows": [_P, _P, _P, _L, _L, _L],
+    "sb_update_weights_noalloc_f32": [_P, _P, _P, _P, _P, _F, _P, _F, _L, _L, _L],
     "sb_net_create": [ctypes.POINTER(_P), _I],
     "sb_net_destroy": [_P],
     "sb_net_add_dense_layer": [_P, _L, _L, _L, _D, _D, _D, _D],

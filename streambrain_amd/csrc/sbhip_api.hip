@@ -34,9 +34,17 @@ struct Context {
   // scratch of the per-kernel training entry points: the "next" Ci / Cj of the fused kernel
   void *trace_next = nullptr;
   long trace_cap = 0;  // elements of 8 bytes
+  // device address of `scratch` on this context's device
+  void *noalloc_scratch = nullptr;
 };
 static Context g_ctx;
 static std::mutex g_ctx_mutex;
+
+// Scratch of sb_update_weights_noalloc_f32: the "next" Ci / Cj of the fused kernel for callers that
+// cannot allocate.  Part of the loaded code object, so every GPU the library runs on holds its own copy
+// until the process ends.  In host code the array's name is only a handle: sb_init asks the runtime for
+// the device address once (g_ctx.noalloc_scratch) and everything below uses that.
+static __device__ __align__(256) unsigned char scratch[SB_NOALLOC_MAX_UNITS * sizeof(float)];
 
 // ---- per-kernel event timing (sb_profile_start / sb_profile_stop)
 struct ProfRecord {
@@ -122,16 +130,18 @@ static int ensure_trace_scratch(long elems) {
 
 // Per-kernel entry points keep the reference's in-place contract: the fused kernel writes the new
 // Ci / Cj into scratch, which is then copied over the caller's arrays.
+// `fixed_scratch`: room for N + M elements that the caller brings (no allocation here), or nullptr to
+// use the context's growable buffer.
 template <typename T>
 static int train_in_place(const T *x, const T *y, T *Cij, T *W, T *Ci, T *Cj, const uint8_t *wmask,
                           int bias_mode, T *bias, T *kbi, long B, long N, long H, long Mc, T taupdt,
-                          T cthr, T khalf, T pmin, T taubdt) {
+                          T cthr, T khalf, T pmin, T taubdt, T *fixed_scratch = nullptr) {
   hipStream_t st = g_ctx.stream;
   const long M = H * Mc;
   SB_REQUIRE(N > 0 && M > 0, "sizes must be positive");
-  int rc = ensure_trace_scratch(N + M);
+  int rc = fixed_scratch ? 0 : ensure_trace_scratch(N + M);
   if (rc) return rc;
-  T *ci_next = (T *)g_ctx.trace_next, *cj_next = ci_next + N;
+  T *ci_next = fixed_scratch ? fixed_scratch : (T *)g_ctx.trace_next, *cj_next = ci_next + N;
   rc = launch_train_fused<T>(st, x, y, Cij, W, Ci, Cj, ci_next, cj_next, wmask, bias_mode, bias, kbi, B,
                              N, H, Mc, taupdt, cthr, khalf, pmin, taubdt, false);
   if (rc) return rc;
@@ -621,7 +631,12 @@ int sb_init(int device) {
     set_error(std::string("sb_init: this library is built for gfx950 only, device is ") + prop.gcnArchName);
     return SB_ERR_UNSUPPORTED;
   }
+  // device address of the static scratch array on this device (the device is current here)
+  void *scratch_ptr = nullptr;
+  SB_HIP(hipGetSymbolAddress(&scratch_ptr, HIP_SYMBOL(scratch)));
+  SB_REQUIRE(scratch_ptr, "no device address for the static scratch array");
   SB_HIP(hipStreamCreate(&g_ctx.stream));
+  g_ctx.noalloc_scratch = scratch_ptr;
   g_ctx.device = device;
   g_ctx.ready = true;
   return 0;
@@ -790,6 +805,27 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
 
 SB_DEFINE_KERNEL_API(f32, float)
 SB_DEFINE_KERNEL_API(f64, double)
+
+// sb_update_weights_f32 for callers that cannot allocate: the new Ci / Cj go through the static scratch
+// array (every element the copies read is written by the kernel first, so nothing needs clearing).  No
+// hipMalloc / hipFree on this path; the event brackets of sb_profile_start would create events, so the
+// call is refused while they are on.
+int sb_update_weights_noalloc_f32(float *Ci, float *Cj, float *Cij, const float *a_i, const float *a_o,
+                                  float taupdt, float *W, float cthr, long B, long N, long M) {
+  SB_READY();
+  SB_REQUIRE(N > 0 && M > 0, "sizes must be positive");
+  if (N + M > (long)SB_NOALLOC_MAX_UNITS) {
+    set_error("sb_update_weights_noalloc_f32: N + M = " + std::to_string(N + M) + " exceeds SB_NOALLOC_MAX_UNITS = " +
+              std::to_string((long)SB_NOALLOC_MAX_UNITS) + "; use sb_update_weights_f32");
+    return SB_ERR_UNSUPPORTED;
+  }
+  if (g_prof_on) {
+    set_error("sb_update_weights_noalloc_f32: not available between sb_profile_start and sb_profile_stop");
+    return SB_ERR_STATE;
+  }
+  return train_in_place<float>(a_i, a_o, Cij, W, Ci, Cj, nullptr, 0, nullptr, nullptr, B, N, 1, M, taupdt, cthr,
+                               0.f, 0.f, 0.f, (float *)g_ctx.noalloc_scratch);
+}
 
 // ================================================================================== C ABI: network
 int sb_net_create(sb_net **net, int dtype) {
