@@ -37,6 +37,16 @@ struct Real<float> {
     const float l2 = __builtin_amdgcn_logf(x * (tiny ? 0x1p32f : 1.0f));
     return __builtin_fmaf(l2, 0.693147180559945309f, tiny ? -32.0f * 0.693147180559945309f : 0.0f);
   }
+  // max(x, floor) for floor >= 0, floor as well when x is NaN; one instruction (the median of x, floor and
+  // +inf; fmax would first quiet a signalling NaN with an instruction of its own)
+  static __device__ __forceinline__ float max_floor(float x, float floor) {
+    return __builtin_amdgcn_fmed3f(x, floor, __builtin_inff());
+  }
+  // the same for arguments known to be at least 2^-96 (bit-identical to wlog there)
+  static __device__ __forceinline__ float wlog_normal(float x) {
+#pragma clang fp contract(off)
+    return __builtin_amdgcn_logf(x) * 0.693147180559945309f;
+  }
   static __device__ __forceinline__ float exp_(float x) { return expf(x); }
   // single IEEE operations: the pragma keeps the compiler from contracting them into FMAs
   static __device__ __forceinline__ float add(float a, float b) {
@@ -64,6 +74,8 @@ struct Real<double> {
   static __device__ __forceinline__ int acc_row(int q, int v) { return 4 * v + q; }
   static __device__ __forceinline__ double log_(double x) { return log(x); }
   static __device__ __forceinline__ double wlog(double x) { return log(x); }
+  static __device__ __forceinline__ double wlog_normal(double x) { return log(x); }
+  static __device__ __forceinline__ double max_floor(double x, double floor) { return fmax(x, floor); }
   static __device__ __forceinline__ double exp_(double x) { return exp(x); }
   static __device__ __forceinline__ double add(double a, double b) {
 #pragma clang fp contract(off)
@@ -142,6 +154,24 @@ struct BufferWindow {
       }
     }
   }
+  // one unconditional 16-byte access at byte offset `at` + `uniform` (kOutside as `at`: no access)
+  __device__ __forceinline__ void load_vec(T (&out)[Real<T>::VW], unsigned at, unsigned uniform) const {
+    const u4 raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)at, (int)uniform, 0);
+    const typename Real<T>::vec_t v = __builtin_bit_cast(typename Real<T>::vec_t, raw);
+#pragma unroll
+    for (int e = 0; e < Real<T>::VW; e++) out[e] = v[e];
+  }
+  // Stores add the uniform offset to the per-lane one and leave the instruction's scalar offset at zero:
+  // the hardware fetches the data registers of a 16-byte store a few cycles after issue, and the compiler
+  // keeps the following instructions from overwriting them only for stores without a scalar offset
+  // register (with one, the first vector instruction after the store clobbered the data of its last lanes
+  // whenever the memory pipeline was busy -- seen on gfx950 as wrong elements 1 and 2 of stored vectors).
+  __device__ __forceinline__ void store_vec(const T (&in)[Real<T>::VW], unsigned at, unsigned uniform) const {
+    typename Real<T>::vec_t v;
+#pragma unroll
+    for (int e = 0; e < Real<T>::VW; e++) v[e] = in[e];
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), rsrc, (int)(at + uniform), 0, 0);
+  }
   // NE consecutive elements (4, 8, 12 or 16 bytes) as one access; element-aligned
   template <int NE>
   __device__ __forceinline__ void load_n(T (&out)[NE], unsigned at) const {
@@ -172,14 +202,14 @@ struct BufferWindow {
 #pragma unroll
       for (int e = 0; e < VW; e++) v[e] = in[e];
       __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), rsrc,
-                                             (int)(col < limit ? at : kOutside), (int)uniform, 0);
+                                             (int)((col < limit ? at : kOutside) + uniform), 0, 0);
     } else if (col + VW <= limit) {
       // (rows that are no whole number of vectors: only the last vector of a row runs over its end, so
       // in all but the last tile column this branch is taken by every lane)
       typename Real<T>::vec_t v;
 #pragma unroll
       for (int e = 0; e < VW; e++) v[e] = in[e];
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), rsrc, (int)at, (int)uniform, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), rsrc, (int)(at + uniform), 0, 0);
     } else {
 #pragma unroll
       for (int e = 0; e < VW; e++) {

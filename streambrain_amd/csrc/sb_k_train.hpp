@@ -8,13 +8,16 @@
 //   bias/kbi <- update_bias_regularized(Cj)                (plastic layers)
 // all from the NEW traces, as the reference's fused loop does.
 //
-// A workgroup (256 threads, 4 wavefronts) owns a 64 x 64 tile of Cij; 16 KiB of LDS and at most 96
+// A workgroup (256 threads, 4 wavefronts) owns a 64 x 64 tile of Cij; 18 KiB of LDS and at most 96
 // registers per thread let five workgroups share a CU, so the 1175 tiles of a 1568 x 3000 layer are
 // all resident at once.
 //   1. Per chunk of KCH batch rows it stages x[:, i-tile] and y[:, j-tile] in LDS.  x and y are
-//      "k-major" in memory, which is the 16x16x4 MFMA operand layout, so staging is a plain copy and
-//      each wavefront feeds its 32 x 32 sub-tile (2 x 2 MFMA blocks) with two 8-byte LDS reads per K
-//      step of 4.  The global loads of chunk c+1 are issued before chunk c is consumed.
+//      "k-major" in memory, which is the 16x16x4 MFMA operand layout, so staging is a plain copy.  Each
+//      wavefront owns 16 rows x 64 columns of the tile (4 MFMA blocks) and feeds them with one element
+//      of x and one 16-byte vector of y per lane and K step of 4; the block columns are interleaved so
+//      that a lane's results of a row are consecutive columns, and the tile is loaded, updated and
+//      stored as 16-byte vectors straight from the accumulator registers (no pass through LDS).  The
+//      global loads of chunk c+1 are issued before chunk c is consumed.
 //   2. From the same LDS slabs, the lanes of one wavefront add up one column each of x, those of
 //      another one column each of y (which two wavefronts rotates with the tile index), in batch order
 //      b = 0..B-1 without FMA contraction: the reference's summation order, so Ci, Cj and kbi stay
@@ -28,18 +31,16 @@
 //      by the time the epilogue needs it.  All loads are branch-free (bounds-checked buffer windows
 //      instead of guards): a guarded load makes the compiler wait for every outstanding load at the
 //      join.
-//   4. The accumulators go through LDS into a row-major layout; each thread then finishes VW consecutive
-//      columns of 4 rows: decay + clamp, weight, mask, one 16-byte store each to Cij and W.  With
-//      w_masked, a wavefront whose vectors of a pass all lie under zero mask bytes skips the weight.
+//   4. Epilogue per 16-byte vector: decay + clamp, weight, mask, one store each to Cij and W.  The
+//      kernel is bound by instruction issue (matrix and vector instructions share the SIMD's issue
+//      slots), so the common case -- no trace of the tile's rows and columns below the threshold, no
+//      logarithm argument near the denormal range, which the two summing wavefronts establish for the
+//      whole tile -- runs a short form of the weight expression (5 vector instructions per synapse), and
+//      with w_masked a wavefront whose vectors all lie under zero mask bytes skips the weight altogether.
 #pragma once
 #include <type_traits>
 
 #include "sb_kernels.hpp"
-
-// Hook for phase timing in development builds; expands to nothing in the library.
-#ifndef SB_PHASE_MARK
-#define SB_PHASE_MARK(n)
-#endif
 
 namespace sb {
 
@@ -59,6 +60,7 @@ struct TrainArgs {
   T *bias, *kbi;
   long B, N, M, H, Mc;
   T tau, omt, fB, invB, cthr, cthr4;
+  T lim;  // traces up to lim (and from cthr) allow the short form of the weight expression, see the kernel
   T khalf, pmin, taubdt;
   long tiles_i, tiles_j;
   FastDiv by_panel, by_Mc;  // divisions by tiles_i * panel_cols and by Mc
@@ -113,9 +115,23 @@ __global__ __launch_bounds__(256) void k_trace_sums(TrainArgs<T> a) {
 }
 
 // Wavefronts per SIMD the registers are budgeted for.  Doubles: four (the LDS slabs allow four workgroups
-// per CU; left alone the compiler takes 176 registers, which allows two).  Floats need no limit: 80-96.
+// per CU; left alone the compiler takes more registers than that allows).  Floats need no limit.
 template <typename T>
 constexpr int train_waves_per_simd() { return sizeof(T) == 8 ? 4 : 1; }
+
+// A raw byte window (for the mask bytes of a tile's rows): bounds-checked like BufferWindow.
+struct ByteWindow {
+  __amdgpu_buffer_rsrc_t rsrc;
+  __device__ ByteWindow(const uint8_t *base, long bytes) {
+    const long b = (base && bytes > 0) ? bytes : 0;
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0,
+                                             (int)(unsigned)(b < 0x80000000L ? b : 0x80000000L), 0x00020000);
+  }
+  __device__ __forceinline__ uint32_t load(unsigned at, unsigned uniform) const {
+    return __builtin_amdgcn_raw_buffer_load_b8(rsrc, (int)at, (int)uniform, 0);
+  }
+};
+
 // VEC: Cij and W are stored as 16-byte vectors (M a multiple of VW), element by element otherwise.  Loads
 // are 16-byte accesses either way: one that runs over the end of a row of x, y or Cij fetches elements of
 // the next row into tile rows / columns outside the matrix, which are never stored or summed.
@@ -127,29 +143,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(train_waves
 void k_train_fused(TrainArgs<T> a) {
   using R = Real<T>;
   using acc_t = typename R::acc_t;
+  using vec_t = typename R::vec_t;
   constexpr int VW = R::VW;             // elements per 16-byte vector
   constexpr int TS = 64;                // tile side
-  constexpr int G = TS / VW;            // 16-byte groups per tile row
-  constexpr int RPP = 256 / G;          // tile rows covered by the workgroup per pass
-  constexpr int PASSES = TS / RPP;      // passes over the tile (epilogue, Cij prefetch)
+  constexpr int G = TS / VW;            // 16-byte groups per slab row
+  constexpr int RPP = 256 / G;          // slab rows the workgroup stages per pass
   constexpr int SP = KCH / RPP;         // staging passes per chunk
-  constexpr int CP = TS + VW;           // pitch of the accumulator tile in LDS
-  // A staged slab row of 64 floats spans the 64 LDS banks exactly, and an 8-byte operand read is served
-  // 32 lanes at a time: lanes (p, q) and (p, q+1), one slab row apart, would meet in the same banks.  Odd
-  // slab rows therefore hold their two halves swapped (column ^ 32).  16-byte reads (doubles) are served
-  // 16 lanes at a time, one slab row: nothing to do.
-  constexpr int SWZ = sizeof(T) == 4 ? 32 : 0;
+  constexpr int NG = 4 / VW;            // 16-byte vectors of a tile row held by one lane
+  // The x slab has a pitch of 80 elements: lane (p, q) of wavefront w reads element 16 w + p of slab row
+  // 4 s + q, and with a pitch of 64 the four q of a column would meet in one LDS bank.
+  constexpr int XP = TS + 16;
+  constexpr int SUMB = 8;               // LDS reads of the column sums in flight at a time
   constexpr bool TILE_IN_LAST = sizeof(T) == 8;  // which chunk requests the Cij tile, see the chunk loop
-  static_assert(RPP % 2 == 0, "row parity of a staging pass");
+  constexpr unsigned ES = sizeof(T);
+  constexpr unsigned kOutside = BufferWindow<T>::kOutside;
   static_assert(KCH % RPP == 0 && KCH % 4 == 0, "chunk size");
-  // LDS: the staging slabs xs | ys; once they are consumed the same memory holds the accumulator tile
-  // followed by the trace reciprocals of the tile's rows and columns
-  constexpr int TAIL = TS * CP + 2 * TS;
-  constexpr int SLAB = 2 * KCH * TS > TAIL ? 2 * KCH * TS : TAIL;
 
-  __shared__ __attribute__((aligned(16))) T slab[SLAB];
-  T *xs = slab, *ys = slab + KCH * TS;
-  T *rci_s = slab + TS * CP, *rcj_s = rci_s + TS;
+  __shared__ __attribute__((aligned(16))) T xs[KCH * XP];
+  __shared__ __attribute__((aligned(16))) T ys[KCH * TS];
+  __shared__ __attribute__((aligned(16))) T rci_s[TS];
+  __shared__ __attribute__((aligned(16))) T rcj_s[TS];
+  __shared__ int slow_s[2];
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, p = lane & 15, q = lane >> 4;
   // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  Renumbered so that one XCD
@@ -164,7 +178,7 @@ void k_train_fused(TrainArgs<T> a) {
   if (tile >= ntiles) return;  // whole workgroup, before any barrier
   const unsigned panel = a.by_panel.div(tile);
   const unsigned in_panel = tile - panel * ((unsigned)a.tiles_i * a.panel_cols);
-  long it = in_panel, jt = panel;
+  unsigned it = in_panel, jt = panel;
   if (a.panel_cols > 1) {  // uniform
     const unsigned first = panel * a.panel_cols;
     const unsigned width = (unsigned)a.tiles_j - first < a.panel_cols ? (unsigned)a.tiles_j - first : a.panel_cols;
@@ -172,40 +186,65 @@ void k_train_fused(TrainArgs<T> a) {
     it = row;
     jt = first + (in_panel - row * width);
   }
-  const long i0 = it * TS, j0 = jt * TS;
+  // every index below fits 32 bits: N, M < 2^31 and 64 rows of x, y, Cij or W stay below 2 GiB (launcher)
+  const unsigned N = (unsigned)a.N, M = (unsigned)a.M;
+  const unsigned i0 = it * TS, j0 = jt * TS;
 
-  // thread's share of the tile in row-major order: VW columns of PASSES rows
-  const int eg = tid % G, er = tid / G;
-  const long ecol = j0 + VW * eg;
-
-  SB_PHASE_MARK(0);
+  // ---- staging: thread (er, eg) copies vector eg of slab rows er, er + RPP, .. of x and of y per chunk.
   // x, y, the Cij tile and the W tile are reached through bounds-checked buffer windows: rows past the
   // batch or past the matrix read zero / store nothing in hardware, so there are no clamped addresses,
-  // no zero-filling and no branches, and the row advance per chunk / pass is a scalar offset.  Loads
-  // return in issue order, hence the order below: first what the first MFMA needs (chunk 0 of x and
-  // y, mostly L2 hits), and the Cij tile (HBM) only while the second-to-last chunk is being computed.
-  constexpr unsigned ES = sizeof(T);
-  const long tile_rows = a.N - i0 < TS ? a.N - i0 : TS;
-  const BufferWindow<T> cwin(a.Cij + i0 * a.M, tile_rows * a.M), wwin(a.W + i0 * a.M, tile_rows * a.M);
+  // no zero-filling and no branches; a vector whose first column lies outside the matrix gets an offset
+  // beyond every window.  Loads return in issue order, hence the order below: first what the first MFMA
+  // needs (chunk 0 of x and y, mostly L2 hits), and the Cij tile (HBM) only late in the chunk loop.
+  const unsigned eg = tid % G, er = tid / G;
+  const unsigned xat = i0 + VW * eg < N ? (er * N + i0 + VW * eg) * ES : kOutside;
+  const unsigned yat = j0 + VW * eg < M ? (er * M + j0 + VW * eg) * ES : kOutside;
+  const unsigned xstep = RPP * N * ES, ystep = RPP * M * ES;  // the next staging pass (uniform)
   T sx[SP][VW], sy[SP][VW];
-  // byte offsets of this thread's vectors relative to the first row of a chunk
-  unsigned xat[SP], yat[SP];
-#pragma unroll
-  for (int m = 0; m < SP; m++) {
-    xat[m] = (unsigned)(((long)(er + RPP * m) * a.N + i0 + VW * eg) * ES);
-    yat[m] = (unsigned)(((long)(er + RPP * m) * a.M + ecol) * ES);
-  }
   auto request_chunk = [&](long b0) {
     // windows from the chunk's first batch row to the end of x / y (scalar arithmetic): rows past the
     // batch fall outside, and the per-lane offsets stay those of chunk 0 whatever the batch size
     const BufferWindow<T> xwin(a.x + b0 * a.N, (a.B - b0) * a.N), ywin(a.y + b0 * a.M, (a.B - b0) * a.M);
 #pragma unroll
     for (int m = 0; m < SP; m++) {
-      xwin.template load<true>(sx[m], xat[m], 0, i0 + VW * eg, a.N);
-      ywin.template load<true>(sy[m], yat[m], 0, ecol, a.M);
+      xwin.load_vec(sx[m], xat, m * xstep);
+      ywin.load_vec(sy[m], yat, m * ystep);
     }
   };
   request_chunk(0);
+
+  // ---- this lane's share of the tile, in the layout the MFMA leaves it in: wavefront w owns tile rows
+  // 16 w .. 16 w + 15 and all 64 columns as four 16 x 16 blocks; the B operand of block c is column
+  // 16 VW (c / VW) + VW p + c % VW, so a lane's VW results of a row are VW consecutive columns: the tile
+  // is loaded, updated and stored as 16-byte vectors straight from the accumulators.  acc[c][v] is row
+  // acc_row(q, v), i.e. rows r0 + rstep v of the wavefront's 16.
+  constexpr int rstep = sizeof(T) == 4 ? 1 : 4;
+  const unsigned r0 = 16 * w + (sizeof(T) == 4 ? 4 * q : q);
+  const long tile_rows = (long)N - i0 < TS ? (long)N - i0 : TS;
+  const BufferWindow<T> cwin(a.Cij + (long)i0 * a.M, tile_rows * a.M), wwin(a.W + (long)i0 * a.M, tile_rows * a.M);
+  unsigned tat[NG], ecol[NG];  // byte offset of row r0 of the lane's vectors inside the windows
+#pragma unroll
+  for (int g = 0; g < NG; g++) {
+    ecol[g] = j0 + 16 * VW * g + VW * p;
+    tat[g] = ecol[g] < M ? (r0 * M + ecol[g]) * ES : kOutside;
+  }
+  const unsigned vstep = rstep * M * ES;  // from acc[..][v] to acc[..][v + 1] (uniform)
+
+  // mask bytes of the lane's synapses: a small, L2-resident array, fetched up front
+  const bool masked = a.wmask != nullptr;
+  uint32_t mb[4][NG][MB];
+  {
+    const ByteWindow mwin(masked ? a.wmask + (long)i0 * a.H : nullptr, tile_rows * a.H);
+    const unsigned H = (unsigned)a.H;
+#pragma unroll
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+      for (int e = 0; e < MB; e++) {
+        const unsigned hc = ecol[g] + e < M ? a.by_Mc.div(ecol[g] + e) : 0u;
+#pragma unroll
+        for (int v = 0; v < 4; v++) mb[v][g][e] = mwin.load(r0 * H + hc, v * rstep * H);
+      }
+  }
 
   // column sums: one wavefront takes the 64 x columns of the tile (a lane each), one the 64 y columns,
   // the other two take none; which wavefronts do rotates with the tile, so that over the tiles of a
@@ -213,10 +252,8 @@ void k_train_fused(TrainArgs<T> a) {
   const int role = __builtin_amdgcn_readfirstlane((w + (int)tile) & 3);
   const bool summer = role < 2;  // uniform per wavefront
   const bool sum_i = role == 0;
-  const int scol = lane;
-  const T *sbase = (sum_i ? xs : ys) + scol, *sbase_odd = (sum_i ? xs : ys) + (scol ^ SWZ);
-  const long sidx = (sum_i ? i0 : j0) + scol;
-  const bool sum_ok = summer && sidx < (sum_i ? a.N : a.M);
+  const unsigned sidx = (sum_i ? i0 : j0) + lane;
+  const bool sum_ok = summer && sidx < (sum_i ? N : M);
   const bool writes_bias = !PRE && sum_ok && !sum_i && it == 0 && a.bias_mode == 1;
   // old trace; with PRE the new one, which the same two wavefronts turn into the reciprocals below
   const T cold = (PRE ? (sum_i ? a.Ci_next : a.Cj_next) : (sum_i ? a.Ci : a.Cj))[sum_ok ? sidx : 0];
@@ -224,89 +261,82 @@ void k_train_fused(TrainArgs<T> a) {
   if (!PRE && a.bias_mode == 1) kb = a.kbi[writes_bias ? sidx : 0];
   T csum = T(0);
 
-  // mask bytes of the thread's PASSES x VW synapses: a small, L2-resident array, fetched up front
-  uint32_t mb[PASSES][MB];
-  if (a.wmask) {
-    uint32_t hc[MB];
-#pragma unroll
-    for (int e = 0; e < MB; e++) hc[e] = ecol + e < a.M ? a.by_Mc.div((uint32_t)(ecol + e)) : 0u;
-#pragma unroll
-    for (int k = 0; k < PASSES; k++) {
-      const long row = i0 + er + RPP * k;
-#pragma unroll
-      for (int e = 0; e < MB; e++) mb[k][e] = a.wmask[row < a.N ? row * a.H + hc[e] : 0];
-    }
-  }
-
-  T cpre[PASSES][VW];  // Cij tile: VW columns of PASSES rows per thread
-  const unsigned tat = (unsigned)(((long)er * a.M + ecol) * ES);  // this thread's vector in pass 0
-  const unsigned pass_bytes = (unsigned)((long)RPP * a.M * ES);    // the next pass is RPP rows further on
+  T cpre[4][NG][VW];  // Cij tile
   auto request_tile = [&]() {
 #pragma unroll
-    for (int k = 0; k < PASSES; k++) cwin.template load<true>(cpre[k], tat, k * pass_bytes, ecol, a.M);
+    for (int v = 0; v < 4; v++)
+#pragma unroll
+      for (int g = 0; g < NG; g++) cwin.load_vec(cpre[v][g], tat[g], v * vstep);
   };
 
-  acc_t acc[2][2];
+  acc_t acc[4];
 #pragma unroll
-  for (int r = 0; r < 2; r++)
-#pragma unroll
-    for (int c = 0; c < 2; c++) acc[r][c] = acc_t{0, 0, 0, 0};
-  const int iw = (w >> 1) * 32, jw = (w & 1) * 32;  // sub-tile of this wavefront
+  for (int c = 0; c < 4; c++) acc[c] = acc_t{0, 0, 0, 0};
 
   // ---- chunks of the batch.  The loads of chunk c+1 are issued before chunk c is consumed from LDS,
   // so their latency hides behind the MFMA loop and the column sums.
   auto chunk = [&](long b0, auto with_tile) {
-    if (b0 > 0) {
-      __syncthreads();  // previous chunk fully consumed
-      SB_PHASE_MARK(2 * (int)(b0 / KCH));
-    }
+    if (b0 > 0) __syncthreads();  // previous chunk fully consumed
 #pragma unroll
     for (int m = 0; m < SP; m++) {
-      typename R::vec_t vx, vy;
+      vec_t vx, vy;
 #pragma unroll
       for (int e = 0; e < VW; e++) {
         vx[e] = sx[m][e];
         vy[e] = sy[m][e];
       }
-      const int at = (er + RPP * m) * TS + ((VW * eg) ^ ((er & 1) * SWZ));
-      *reinterpret_cast<typename R::vec_t *>(&xs[at]) = vx;
-      *reinterpret_cast<typename R::vec_t *>(&ys[at]) = vy;
+      *reinterpret_cast<vec_t *>(&xs[(er + RPP * m) * XP + VW * eg]) = vx;
+      *reinterpret_cast<vec_t *>(&ys[(er + RPP * m) * TS + VW * eg]) = vy;
     }
     __syncthreads();
-    SB_PHASE_MARK(1 + 2 * (int)(b0 / KCH));
     request_chunk(b0 + KCH);  // past the batch: reads zeros nobody consumes
     if (decltype(with_tile)::value) request_tile();
 
     if (!PRE && summer) {
-      // rows past the end of the batch were staged as zeros: adding them changes nothing, so the loop
-      // needs no guard; 16 LDS reads are in flight before the (ordered) additions consume them
-      for (int r = 0; r < KCH; r += 16) {
-        T v[16];
+      // rows past the end of the batch were staged as zeros: adding them changes nothing, so the loops
+      // need no guard; SUMB LDS reads are in flight before the (ordered) additions consume them
+      // (two copies so that the slab pitch is a constant and the reads take immediate offsets)
+      if (sum_i) {
+        for (int r = 0; r < KCH; r += SUMB) {
+          T v[SUMB];
 #pragma unroll
-        for (int k = 0; k < 16; k++) v[k] = (k & 1 ? sbase_odd : sbase)[(r + k) * TS];
+          for (int k = 0; k < SUMB; k++) v[k] = xs[(r + k) * XP + lane];
 #pragma unroll
-        for (int k = 0; k < 16; k++) csum = R::add(csum, v[k]);
+          for (int k = 0; k < SUMB; k++) csum = R::add(csum, v[k]);
+        }
+      } else {
+        for (int r = 0; r < KCH; r += SUMB) {
+          T v[SUMB];
+#pragma unroll
+          for (int k = 0; k < SUMB; k++) v[k] = ys[(r + k) * TS + lane];
+#pragma unroll
+          for (int k = 0; k < SUMB; k++) csum = R::add(csum, v[k]);
+        }
       }
     }
 
-    // K loop: per step of 4 batch rows, lane (p,q) feeds row 4s+q of the slabs.  The operands of step
-    // s+1 are read from LDS before the MFMAs of step s are issued (the fences keep that order).
-    const T *xa = xs + q * TS + ((iw + 2 * p) ^ ((q & 1) * SWZ));
-    const T *ya = ys + q * TS + ((jw + 2 * p) ^ ((q & 1) * SWZ));
-    T xo[2][2], yo[2][2];
-    xo[0][0] = xa[0], xo[0][1] = xa[1], yo[0][0] = ya[0], yo[0][1] = ya[1];
+    // K loop: per step of 4 batch rows, lane (p, q) feeds slab row 4 s + q: one element of x, NG vectors
+    // of y.  The operands of step s+1 are read from LDS before the MFMAs of step s are issued (the
+    // fences keep that order).
+    const T *xa = xs + q * XP + 16 * w + p;
+    const T *ya = ys + q * TS + VW * p;
+    T xo[2];
+    vec_t yo[2][NG];
+    xo[0] = xa[0];
+#pragma unroll
+    for (int g = 0; g < NG; g++) yo[0][g] = *reinterpret_cast<const vec_t *>(ya + 16 * VW * g);
 #pragma unroll
     for (int s = 0; s < KCH / 4; s++) {
       const int cur = s & 1, nxt = cur ^ 1;
       if (s + 1 < KCH / 4) {
-        xo[nxt][0] = xa[(s + 1) * 4 * TS], xo[nxt][1] = xa[(s + 1) * 4 * TS + 1];
-        yo[nxt][0] = ya[(s + 1) * 4 * TS], yo[nxt][1] = ya[(s + 1) * 4 * TS + 1];
+        xo[nxt] = xa[(s + 1) * 4 * XP];
+#pragma unroll
+        for (int g = 0; g < NG; g++)
+          yo[nxt][g] = *reinterpret_cast<const vec_t *>(ya + (s + 1) * 4 * TS + 16 * VW * g);
       }
       __builtin_amdgcn_sched_barrier(0);
-      acc[0][0] = R::mfma(xo[cur][0], yo[cur][0], acc[0][0]);
-      acc[0][1] = R::mfma(xo[cur][0], yo[cur][1], acc[0][1]);
-      acc[1][0] = R::mfma(xo[cur][1], yo[cur][0], acc[1][0]);
-      acc[1][1] = R::mfma(xo[cur][1], yo[cur][1], acc[1][1]);
+#pragma unroll
+      for (int c = 0; c < 4; c++) acc[c] = R::mfma(xo[cur], yo[cur][c / VW][c % VW], acc[c]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -323,12 +353,13 @@ void k_train_fused(TrainArgs<T> a) {
     if (b0 < a.B) chunk(b0, std::false_type{});
   }
 
-  __syncthreads();  // slabs consumed: their memory is reused from here on
-  SB_PHASE_MARK(12);
-
-  // ---- 3. new traces of this tile's rows and columns (reference order of operations)
+  // ---- new traces of this tile's rows and columns (reference order of operations), their reciprocals
+  // for the weights, and whether the tile can take the short form of the weight expression: every row
+  // and column trace at or above the threshold (no weight forced to zero) and small enough that no
+  // argument of the logarithm can fall below 2^-96 (max(Cij, cthr^4) / (Ci Cj) >= cthr^4 / lim^2).
   if (summer) {
     T cnew = T(1);
+    bool odd = false;
     if (sum_ok) {
       if constexpr (PRE) {
         cnew = cold;
@@ -344,63 +375,83 @@ void k_train_fused(TrainArgs<T> a) {
           }
         }
       }
+      odd = !(cnew >= a.cthr) || !(cnew <= a.lim);
     }
-    (sum_i ? rci_s : rcj_s)[scol] = trace_reciprocal<T>(cnew, a.cthr);
+    (sum_i ? rci_s : rcj_s)[lane] = trace_reciprocal<T>(cnew, a.cthr);
+    if (lane == 0) slow_s[role] = 0;
+    if (odd) slow_s[role] = 1;
   }
+  __syncthreads();  // reciprocals and flags published
 
-  // ---- 4. accumulators -> row-major LDS tile
-  T *cs = slab;
-#pragma unroll
-  for (int r = 0; r < 2; r++)
-#pragma unroll
-    for (int v = 0; v < 4; v++) {
-      const int row = iw + 2 * R::acc_row(q, v) + r;
-      cs[row * CP + jw + 2 * p] = acc[r][0][v];
-      cs[row * CP + jw + 2 * p + 1] = acc[r][1][v];
-    }
-  __syncthreads();  // accumulator tile and reciprocals published
-  SB_PHASE_MARK(13);
-
-  // ---- epilogue: decay + clamp, weight, mask, stores.  Whether a synapse keeps its weight (row and
-  // column above the trace threshold, mask bit set) is combined into one predicate per element.
+  // ---- epilogue: decay + clamp, weight, mask, stores
   const T scale = a.invB * a.tau;
-  const bool masked = a.wmask != nullptr;
-  T rcj[VW];
-  bool col_live[VW];
+  T rci[4];
+  vec_t rcj[NG];
 #pragma unroll
-  for (int e = 0; e < VW; e++) {
-    rcj[e] = rcj_s[VW * eg + e];
-    col_live[e] = !(rcj[e] < T(0));
+  for (int v = 0; v < 4; v++) rci[v] = rci_s[r0 + rstep * v];
+#pragma unroll
+  for (int g = 0; g < NG; g++) rcj[g] = *reinterpret_cast<const vec_t *>(&rcj_s[16 * VW * g + VW * p]);
+  const bool slow = __builtin_amdgcn_readfirstlane(slow_s[0] | slow_s[1]) != 0;
+
+  if (VEC && MB == 1 && !slow) {
+    // short form: no row or column is dead, no argument is tiny; a vector lies in one hypercolumn
+#pragma unroll
+    for (int v = 0; v < 4; v++)
+#pragma unroll
+      for (int g = 0; g < NG; g++) {
+        T cn[VW], cv[VW];
+#pragma unroll
+        for (int e = 0; e < VW; e++) {
+          cn[e] = cpre[v][g][e] * a.omt + acc[g * VW + e][v] * scale;
+          cv[e] = fmax(cn[e], T(0));  // 0 as well when cn is NaN, like the reference's `cn > 0 ? cn : 0`
+        }
+        cwin.store_vec(cv, tat[g], v * vstep);
+        if (a.W == nullptr) continue;
+        // Where the mask is 0 the weight is 0, and when the caller vouches that W holds 0 there already,
+        // such vectors are not stored, and a wavefront without a connected vector computes nothing.
+        const bool connected = !masked || mb[v][g][0] != 0;
+        if (a.w_masked && __builtin_amdgcn_ballot_w64(connected) == 0) continue;
+        T wv[VW];
+#pragma unroll
+        // (max(max(cn, 0), cthr^4) = max(cn, cthr^4), cthr^4 as well when cn is NaN)
+        for (int e = 0; e < VW; e++) wv[e] = R::wlog_normal(R::max_floor(cn[e], a.cthr4) * rci[v] * rcj[g][e]);
+        if (!a.w_masked) {  // uniform
+#pragma unroll
+          for (int e = 0; e < VW; e++) wv[e] = connected ? wv[e] : T(0);
+        }
+        wwin.store_vec(wv, (a.w_masked && !connected) ? kOutside : tat[g], v * vstep);
+      }
+    return;
   }
+
+  // general form: whether a synapse keeps its weight (row and column above the trace threshold, mask
+  // bit set) is combined into one predicate per element
 #pragma unroll
-  for (int k = 0; k < PASSES; k++) {
-    const int lr = er + RPP * k;  // rows past the matrix compute garbage that the window drops
-    const T rci = rci_s[lr];
-    const bool row_live = !(rci < T(0)) && (MB != 1 || !masked || mb[k][0] != 0);
-    T cv[VW];
+  for (int v = 0; v < 4; v++)
 #pragma unroll
-    for (int e = 0; e < VW; e++) {
-      const T cn = cpre[k][e] * a.omt + cs[lr * CP + VW * eg + e] * scale;
-      cv[e] = fmax(cn, T(0));  // 0 as well when cn is NaN, like the reference's `cn > 0 ? cn : 0`
+    for (int g = 0; g < NG; g++) {
+      const bool row_live = !(rci[v] < T(0)) && (MB != 1 || !masked || mb[v][g][0] != 0);
+      T cv[VW];
+#pragma unroll
+      for (int e = 0; e < VW; e++) {
+        const T cn = cpre[v][g][e] * a.omt + acc[g * VW + e][v] * scale;
+        cv[e] = fmax(cn, T(0));
+      }
+      cwin.template store<VEC>(cv, tat[g], v * vstep, ecol[g], a.M);
+      bool connected = !masked;
+#pragma unroll
+      for (int e = 0; e < MB; e++) connected = connected || mb[v][g][e] != 0;
+      if (a.W == nullptr) continue;
+      if (a.w_masked && __builtin_amdgcn_ballot_w64(connected) == 0) continue;
+      T wv[VW];
+#pragma unroll
+      for (int e = 0; e < VW; e++) {
+        const T wgt = R::wlog(fmax(cv[e], a.cthr4) * rci[v] * rcj[g][e]);
+        const bool keep = row_live && !(rcj[g][e] < T(0)) && (MB == 1 || !masked || mb[v][g][e] != 0);
+        wv[e] = keep ? wgt : T(0);
+      }
+      wwin.template store<VEC>(wv, tat[g], v * vstep, ecol[g], a.M);
     }
-    cwin.template store<VEC>(cv, tat, k * pass_bytes, ecol, a.M);
-    // Where the mask is 0 the weight is 0, and when the caller vouches that W holds 0 there already, a
-    // wavefront whose vectors all lie under zero mask bytes has nothing to compute or store.
-    bool connected = !masked;
-#pragma unroll
-    for (int e = 0; e < MB; e++) connected = connected || mb[k][e] != 0;
-    if (a.W == nullptr) continue;
-    if (a.w_masked && __builtin_amdgcn_ballot_w64(connected) == 0) continue;
-    T wv[VW];
-#pragma unroll
-    for (int e = 0; e < VW; e++) {
-      const T wgt = R::wlog(fmax(cv[e], a.cthr4) * rci * rcj[e]);
-      const bool keep = row_live && col_live[e] && (MB == 1 || !masked || mb[k][e] != 0);
-      wv[e] = keep ? wgt : T(0);
-    }
-    wwin.template store<VEC>(wv, tat, k * pass_bytes, ecol, a.M);
-  }
-  SB_PHASE_MARK(14);
 }
 
 }  // namespace sb

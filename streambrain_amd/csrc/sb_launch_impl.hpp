@@ -252,6 +252,10 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   a.bias_mode = bias_mode; a.bias = bias; a.kbi = kbi;
   a.B = B; a.N = N; a.M = M; a.H = H; a.Mc = Mc;
   a.tau = s.tau; a.omt = s.omt; a.fB = (T)B; a.invB = (T)1 / (T)B; a.cthr = s.cthr; a.cthr4 = s.cthr4;
+  // traces up to cthr^2 * 2^48 keep every argument max(Cij, cthr^4) / (Ci Cj) of the float weight
+  // logarithm at or above 2^-96; doubles have no such limit
+  if constexpr (sizeof(T) == 4) a.lim = s.cthr * s.cthr * 0x1p48f;
+  else a.lim = (T)INFINITY;
   a.khalf = khalf; a.pmin = pmin; a.taubdt = taubdt;
   a.tiles_i = cdiv(N, 64); a.tiles_j = cdiv(M, 64);
   // tile order (see the kernel): column-major while a batch of x fits an L2 with room to spare, panels of
