@@ -126,6 +126,11 @@ struct BufferWindow {
     // descriptor word 3 = 0x00020000: raw buffer, 32-bit data format, as for every untyped gfx9 buffer
     rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(base), 0, (int)size, 0x00020000);
   }
+  // the same for a caller that has the size in bytes at hand (at most 2 GiB)
+  struct Bytes { unsigned n; };
+  __device__ BufferWindow(const T *base, Bytes bytes) {
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(base), 0, (int)bytes.n, 0x00020000);
+  }
   using u4 = unsigned __attribute__((ext_vector_type(4)));
   using u2 = unsigned __attribute__((ext_vector_type(2)));
   // `at`: byte offset of the vector's first element (ignored parts: see `col`, `limit`); VEC moves the

@@ -172,19 +172,22 @@ void k_train_fused(TrainArgs<T> a) {
   // limited set of row slabs of x.  One column per panel (column-major order) when the whole batch of x
   // fits an L2 anyway: a few hundred KB of y plus all of x per L2.  For big layers a column-major order
   // re-read x from HBM once per tile column (measured 460 GB per launch at 65536 x 100000, batch 1024).
-  const unsigned ntiles = (unsigned)(a.tiles_i * a.tiles_j);  // < 2^31, checked by the launcher
-  const unsigned per_xcd = (ntiles + 7) / 8;
-  const unsigned tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (tile >= ntiles) return;  // whole workgroup, before any barrier
-  const unsigned panel = a.by_panel.div(tile);
-  const unsigned in_panel = tile - panel * ((unsigned)a.tiles_i * a.panel_cols);
-  unsigned it = in_panel, jt = panel;
-  if (a.panel_cols > 1) {  // uniform
+  // The grid has one workgroup per tile; XCD x = blockIdx % 8 holds tiles_of(x) = ntiles / 8 (+1 for
+  // x < ntiles % 8) consecutive tiles.
+  const unsigned ntiles = (unsigned)a.tiles_i * (unsigned)a.tiles_j;  // < 2^31, checked by the launcher
+  const unsigned xcd = blockIdx.x & 7, rem = ntiles & 7;
+  const unsigned tile = xcd * (ntiles >> 3) + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3);
+  unsigned it, jt;
+  if (a.panel_cols == 1) {  // uniform
+    jt = a.by_panel.div(tile);
+    it = tile - jt * (unsigned)a.tiles_i;
+  } else {
+    const unsigned panel = a.by_panel.div(tile);
+    const unsigned in_panel = tile - panel * ((unsigned)a.tiles_i * a.panel_cols);
     const unsigned first = panel * a.panel_cols;
     const unsigned width = (unsigned)a.tiles_j - first < a.panel_cols ? (unsigned)a.tiles_j - first : a.panel_cols;
-    const unsigned row = width == a.panel_cols ? in_panel >> __builtin_ctz(a.panel_cols) : in_panel / width;
-    it = row;
-    jt = first + (in_panel - row * width);
+    it = width == a.panel_cols ? in_panel >> __builtin_ctz(a.panel_cols) : in_panel / width;
+    jt = first + (in_panel - it * width);
   }
   // every index below fits 32 bits: N, M < 2^31 and 64 rows of x, y, Cij or W stay below 2 GiB (launcher)
   const unsigned N = (unsigned)a.N, M = (unsigned)a.M;
@@ -201,17 +204,25 @@ void k_train_fused(TrainArgs<T> a) {
   const unsigned yat = j0 + VW * eg < M ? (er * M + j0 + VW * eg) * ES : kOutside;
   const unsigned xstep = RPP * N * ES, ystep = RPP * M * ES;  // the next staging pass (uniform)
   T sx[SP][VW], sy[SP][VW];
-  auto request_chunk = [&](long b0) {
-    // windows from the chunk's first batch row to the end of x / y (scalar arithmetic): rows past the
-    // batch fall outside, and the per-lane offsets stay those of chunk 0 whatever the batch size
-    const BufferWindow<T> xwin(a.x + b0 * a.N, (a.B - b0) * a.N), ywin(a.y + b0 * a.M, (a.B - b0) * a.M);
+  // Windows over the rows of one chunk: rows past the batch fall outside, and the per-lane offsets stay
+  // those of chunk 0 whatever the batch size.  The chunk's first row advances by pointer; sizes are
+  // 32-bit (KCH rows of x or y stay below 2 GiB).
+  const T *xnext = a.x, *ynext = a.y;
+  unsigned rows_left = (unsigned)a.B;  // B < 2^31 (launcher)
+  auto request_chunk = [&]() {
+    const unsigned rows = rows_left < (unsigned)KCH ? rows_left : (unsigned)KCH;
+    const BufferWindow<T> xwin(xnext, typename BufferWindow<T>::Bytes{rows * N * ES}),
+        ywin(ynext, typename BufferWindow<T>::Bytes{rows * M * ES});
 #pragma unroll
     for (int m = 0; m < SP; m++) {
       xwin.load_vec(sx[m], xat, m * xstep);
       ywin.load_vec(sy[m], yat, m * ystep);
     }
+    xnext += KCH * N;
+    ynext += KCH * M;
+    rows_left -= rows;
   };
-  request_chunk(0);
+  request_chunk();
 
   // ---- this lane's share of the tile, in the layout the MFMA leaves it in: wavefront w owns tile rows
   // 16 w .. 16 w + 15 and all 64 columns as four 16 x 16 blocks; the B operand of block c is column
@@ -221,7 +232,9 @@ void k_train_fused(TrainArgs<T> a) {
   constexpr int rstep = sizeof(T) == 4 ? 1 : 4;
   const unsigned r0 = 16 * w + (sizeof(T) == 4 ? 4 * q : q);
   const long tile_rows = (long)N - i0 < TS ? (long)N - i0 : TS;
-  const BufferWindow<T> cwin(a.Cij + (long)i0 * a.M, tile_rows * a.M), wwin(a.W + (long)i0 * a.M, tile_rows * a.M);
+  const unsigned tile_bytes = (unsigned)tile_rows * M * ES;  // at most 2 GiB (launcher)
+  const BufferWindow<T> cwin(a.Cij + (long)i0 * a.M, typename BufferWindow<T>::Bytes{tile_bytes}),
+      wwin(a.W + (long)i0 * a.M, typename BufferWindow<T>::Bytes{a.W ? tile_bytes : 0u});
   unsigned tat[NG], ecol[NG];  // byte offset of row r0 of the lane's vectors inside the windows
 #pragma unroll
   for (int g = 0; g < NG; g++) {
@@ -289,7 +302,7 @@ void k_train_fused(TrainArgs<T> a) {
       *reinterpret_cast<vec_t *>(&ys[(er + RPP * m) * TS + VW * eg]) = vy;
     }
     __syncthreads();
-    request_chunk(b0 + KCH);  // past the batch: reads zeros nobody consumes
+    request_chunk();  // the next one; past the batch: reads zeros nobody consumes
     if (decltype(with_tile)::value) request_tile();
 
     if (!PRE && summer) {

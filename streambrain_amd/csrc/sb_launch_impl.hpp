@@ -244,7 +244,7 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   SB_REQUIRE(bias_mode == 0 || (bias && kbi), "bias update needs bias and kbi");
   SB_REQUIRE(B > 0 && N > 0 && H > 0 && Mc > 0, "sizes must be positive");
   const long M = H * Mc;
-  SB_REQUIRE(M < (1L << 31) && N < (1L << 31), "dimension too large");
+  SB_REQUIRE(M < (1L << 31) && N < (1L << 31) && B < (1L << 31), "dimension too large");
   const TraceScalars<T> s = TraceScalars<T>::from(taupdt, cthr);
   TrainArgs<T> a;
   a.x = x; a.y = y; a.Cij = Cij; a.W = W; a.Ci = Ci; a.Cj = Cj; a.Ci_next = Ci_next; a.Cj_next = Cj_next;
@@ -284,9 +284,8 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   // 16-byte stores of Cij and W need rows that are whole vectors (a vector must not run into the next
   // row); loads are 16-byte accesses for every shape, and neither needs more than element alignment
   const bool vec = M % VW == 0;
-  // 8 workgroup ids per round of XCDs; ids beyond the last tile exit at once
-  const dim3 grid((unsigned)(8 * cdiv(a.tiles_i * a.tiles_j, 8)));
-  // batch rows staged per chunk: 16 KiB of LDS per workgroup, so five workgroups share a CU
+  const dim3 grid((unsigned)(a.tiles_i * a.tiles_j));  // one workgroup per tile
+  // batch rows staged per chunk: 18 KiB of LDS per workgroup, so five workgroups share a CU
   constexpr int KCH = 32;
   const bool one_byte = Mc % VW == 0;  // every vector of VW columns lies inside one hypercolumn
   ProfScope prof_(st, K_TRAIN_FUSED);
