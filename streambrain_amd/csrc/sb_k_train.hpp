@@ -286,6 +286,35 @@ void k_train_fused(TrainArgs<T> a) {
 #pragma unroll
   for (int c = 0; c < 4; c++) acc[c] = acc_t{0, 0, 0, 0};
 
+  // ---- new traces of this tile's rows and columns (reference order of operations), their reciprocals
+  // for the weights, and whether the tile can take the short form of the weight expression: every row
+  // and column trace at or above the threshold (no weight forced to zero) and small enough that no
+  // argument of the logarithm can fall below 2^-96 (max(Cij, cthr^4) / (Ci Cj) >= cthr^4 / lim^2).
+  auto finish_traces = [&]() {
+    T cnew = T(1);
+    bool odd = false;
+    if (sum_ok) {
+      if constexpr (PRE) {
+        cnew = cold;
+      } else {
+        cnew = trace_next<T>(cold, csum, a);
+        if (sum_i) {
+          if (jt == 0) a.Ci_next[sidx] = cnew;
+        } else if (it == 0) {
+          a.Cj_next[sidx] = cnew;
+          if (writes_bias) {
+            a.bias[sidx] = bias_regularized<T>(cnew, kb, a.cthr, a.khalf, a.pmin, a.taubdt);
+            a.kbi[sidx] = kb;
+          }
+        }
+      }
+      odd = !(cnew >= a.cthr) || !(cnew <= a.lim);
+    }
+    (sum_i ? rci_s : rcj_s)[lane] = trace_reciprocal<T>(cnew, a.cthr);
+    if (lane == 0) slow_s[role] = 0;
+    if (odd) slow_s[role] = 1;
+  };
+
   // ---- chunks of the batch.  The loads of chunk c+1 are issued before chunk c is consumed from LDS,
   // so their latency hides behind the MFMA loop and the column sums.
   auto chunk = [&](long b0, auto with_tile) {
@@ -328,6 +357,10 @@ void k_train_fused(TrainArgs<T> a) {
       }
     }
 
+    // after the last chunk's sums the new traces are complete: the two summing wavefronts turn them into
+    // reciprocals for the weights while the others are still multiplying
+    if (summer && b0 + KCH >= a.B) finish_traces();
+
     // K loop: per step of 4 batch rows, lane (p, q) feeds slab row 4 s + q: one element of x, NG vectors
     // of y.  The operands of step s+1 are read from LDS before the MFMAs of step s are issued (the
     // fences keep that order).
@@ -366,38 +399,26 @@ void k_train_fused(TrainArgs<T> a) {
     if (b0 < a.B) chunk(b0, std::false_type{});
   }
 
-  // ---- new traces of this tile's rows and columns (reference order of operations), their reciprocals
-  // for the weights, and whether the tile can take the short form of the weight expression: every row
-  // and column trace at or above the threshold (no weight forced to zero) and small enough that no
-  // argument of the logarithm can fall below 2^-96 (max(Cij, cthr^4) / (Ci Cj) >= cthr^4 / lim^2).
-  if (summer) {
-    T cnew = T(1);
-    bool odd = false;
-    if (sum_ok) {
-      if constexpr (PRE) {
-        cnew = cold;
-      } else {
-        cnew = trace_next<T>(cold, csum, a);
-        if (sum_i) {
-          if (jt == 0) a.Ci_next[sidx] = cnew;
-        } else if (it == 0) {
-          a.Cj_next[sidx] = cnew;
-          if (writes_bias) {
-            a.bias[sidx] = bias_regularized<T>(cnew, kb, a.cthr, a.khalf, a.pmin, a.taubdt);
-            a.kbi[sidx] = kb;
-          }
-        }
-      }
-      odd = !(cnew >= a.cthr) || !(cnew <= a.lim);
-    }
-    (sum_i ? rci_s : rcj_s)[lane] = trace_reciprocal<T>(cnew, a.cthr);
-    if (lane == 0) slow_s[role] = 0;
-    if (odd) slow_s[role] = 1;
-  }
-  __syncthreads();  // reciprocals and flags published
-
-  // ---- epilogue: decay + clamp, weight, mask, stores
+  // ---- epilogue: decay + clamp and the Cij stores first (they need nothing from the other wavefronts),
+  // then, once the reciprocals are published, weight, mask and the W stores
   const T scale = a.invB * a.tau;
+  T cn[4][NG][VW];
+#pragma unroll
+  for (int v = 0; v < 4; v++)
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+      T cv[VW];
+#pragma unroll
+      for (int e = 0; e < VW; e++) {
+        cn[v][g][e] = cpre[v][g][e] * a.omt + acc[g * VW + e][v] * scale;
+        cv[e] = fmax(cn[v][g][e], T(0));  // 0 as well when cn is NaN, like the reference's `cn > 0 ? cn : 0`
+      }
+      if (VEC) cwin.store_vec(cv, tat[g], v * vstep);
+      else cwin.template store<false>(cv, tat[g], v * vstep, ecol[g], a.M);
+    }
+  if (a.W == nullptr) return;  // (uniform) traces only
+
+  __syncthreads();  // reciprocals and flags published
   T rci[4];
   vec_t rcj[NG];
 #pragma unroll
@@ -407,27 +428,20 @@ void k_train_fused(TrainArgs<T> a) {
   const bool slow = __builtin_amdgcn_readfirstlane(slow_s[0] | slow_s[1]) != 0;
 
   if (VEC && MB == 1 && !slow) {
-    // short form: no row or column is dead, no argument is tiny; a vector lies in one hypercolumn
+    // short form: no row or column is dead, no argument is tiny; a vector lies in one hypercolumn.
+    // Where the mask is 0 the weight is 0, and when the caller vouches that W holds 0 there already,
+    // such vectors are not stored, and a wavefront without a connected vector computes nothing.
 #pragma unroll
     for (int v = 0; v < 4; v++)
 #pragma unroll
       for (int g = 0; g < NG; g++) {
-        T cn[VW], cv[VW];
-#pragma unroll
-        for (int e = 0; e < VW; e++) {
-          cn[e] = cpre[v][g][e] * a.omt + acc[g * VW + e][v] * scale;
-          cv[e] = fmax(cn[e], T(0));  // 0 as well when cn is NaN, like the reference's `cn > 0 ? cn : 0`
-        }
-        cwin.store_vec(cv, tat[g], v * vstep);
-        if (a.W == nullptr) continue;
-        // Where the mask is 0 the weight is 0, and when the caller vouches that W holds 0 there already,
-        // such vectors are not stored, and a wavefront without a connected vector computes nothing.
         const bool connected = !masked || mb[v][g][0] != 0;
         if (a.w_masked && __builtin_amdgcn_ballot_w64(connected) == 0) continue;
         T wv[VW];
 #pragma unroll
         // (max(max(cn, 0), cthr^4) = max(cn, cthr^4), cthr^4 as well when cn is NaN)
-        for (int e = 0; e < VW; e++) wv[e] = R::wlog_normal(R::max_floor(cn[e], a.cthr4) * rci[v] * rcj[g][e]);
+        for (int e = 0; e < VW; e++)
+          wv[e] = R::wlog_normal(R::max_floor(cn[v][g][e], a.cthr4) * rci[v] * rcj[g][e]);
         if (!a.w_masked) {  // uniform
 #pragma unroll
           for (int e = 0; e < VW; e++) wv[e] = connected ? wv[e] : T(0);
@@ -444,22 +458,14 @@ void k_train_fused(TrainArgs<T> a) {
 #pragma unroll
     for (int g = 0; g < NG; g++) {
       const bool row_live = !(rci[v] < T(0)) && (MB != 1 || !masked || mb[v][g][0] != 0);
-      T cv[VW];
-#pragma unroll
-      for (int e = 0; e < VW; e++) {
-        const T cn = cpre[v][g][e] * a.omt + acc[g * VW + e][v] * scale;
-        cv[e] = fmax(cn, T(0));
-      }
-      cwin.template store<VEC>(cv, tat[g], v * vstep, ecol[g], a.M);
       bool connected = !masked;
 #pragma unroll
       for (int e = 0; e < MB; e++) connected = connected || mb[v][g][e] != 0;
-      if (a.W == nullptr) continue;
       if (a.w_masked && __builtin_amdgcn_ballot_w64(connected) == 0) continue;
       T wv[VW];
 #pragma unroll
       for (int e = 0; e < VW; e++) {
-        const T wgt = R::wlog(fmax(cv[e], a.cthr4) * rci[v] * rcj[g][e]);
+        const T wgt = R::wlog(R::max_floor(cn[v][g][e], a.cthr4) * rci[v] * rcj[g][e]);
         const bool keep = row_live && !(rcj[g][e] < T(0)) && (MB == 1 || !masked || mb[v][g][e] != 0);
         wv[e] = keep ? wgt : T(0);
       }
