@@ -38,7 +38,23 @@ def one_hot_labels(rng, n, n_classes):
     return lab
 
 
-def rel_err(a, ref):
+def rel_err(a, ref, what=None, tol=float("nan")):
+    """max |a - ref| / max(|ref|, 1); with `what`, the value is also recorded for the measured-error table."""
     a = np.asarray(a, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)
-    return float(np.max(np.abs(a - ref) / np.maximum(np.abs(ref), 1.0))) if a.size else 0.0
+    e = float(np.max(np.abs(a - ref) / np.maximum(np.abs(ref), 1.0))) if a.size else 0.0
+    if what is not None:
+        record_error(what, e, tol)
+    return e
+
+
+# Measured parity errors of the GPU tests, by test id and quantity: (error, tolerance asserted).  The
+# session hook in conftest.py writes them out, so the bound a test asserts can be compared with what was
+# measured.
+MEASURED = {}
+
+
+def record_error(what, e, tol):
+    import os
+    test = os.environ.get("PYTEST_CURRENT_TEST", "?").split(" ")[0]
+    MEASURED.setdefault(test, []).append((what, float(e), float(tol)))

@@ -6,6 +6,8 @@ import ctypes
 import numpy as np
 import pytest
 
+from helpers import record_error
+
 pytestmark = pytest.mark.gpu
 
 
@@ -88,8 +90,12 @@ def _check_layer_at_size(dtype, B, N, H, Mc, density, seed):
         cij_row = _slice_to_host(_capi, lib, d_cij, i * M, M, dtype)
         w_row = _slice_to_host(_capi, lib, d_w, i * M, M, dtype)
         ref_cij, ref_w = weights_of(i, every)
-        assert np.max(np.abs(cij_row - ref_cij) / np.maximum(np.abs(ref_cij), 1)) <= tol, f"Cij row {i}"
-        assert np.max(np.abs(w_row - ref_w) / np.maximum(np.abs(ref_w), 1)) <= 2 * tol, f"W row {i}"
+        e_cij = np.max(np.abs(cij_row - ref_cij) / np.maximum(np.abs(ref_cij), 1))
+        e_w = np.max(np.abs(w_row - ref_w) / np.maximum(np.abs(ref_w), 1))
+        record_error(f"Cij row {i}", e_cij, tol)
+        record_error(f"W row {i}", e_w, tol)
+        assert e_cij <= tol, f"Cij row {i}"
+        assert e_w <= tol, f"W row {i}"
 
     # forward through the trained, masked W: one hypercolumn against the host (its W columns read back
     # for the connected rows and checked against the closed form), all of it dense kernel against
@@ -101,7 +107,7 @@ def _check_layer_at_size(dtype, B, N, H, Mc, density, seed):
     sample = connected[:: max(1, len(connected) // 2000)]
     got_w = _rows_to_host(_capi, lib, d_w, sample, M, h * Mc, Mc, dtype)
     for k in range(0, len(sample), max(1, len(sample) // 16)):
-        assert np.max(np.abs(got_w[k] - weights_of(sample[k], cols)[1])) <= 2 * tol * 30
+        assert np.max(np.abs(got_w[k] - weights_of(sample[k], cols)[1])) <= tol * 30
     bs = [0, B // 2, B - 1]
     terms = float((x[bs][:, sample].astype(np.float64) @ np.abs(got_w).astype(np.float64)).max())
     terms *= len(connected) / len(sample)
@@ -115,7 +121,8 @@ def _check_layer_at_size(dtype, B, N, H, Mc, density, seed):
         logits = xs[bs][:, connected].astype(np.float64) @ got_w.astype(np.float64) + bias[cols]
         e = np.exp(logits - logits.max(axis=1, keepdims=True))
         ref = e / e.sum(axis=1, keepdims=True)
-        assert np.max(np.abs(act[bs][:, cols] - ref)) <= 16 * tol
+        record_error("activation vs host", np.max(np.abs(act[bs][:, cols] - ref)), tol)
+        assert np.max(np.abs(act[bs][:, cols] - ref)) <= tol
     if density <= 0.5:
         cap = (int(np.count_nonzero(wmask, axis=0).max()) + 15) // 16 * 16 + 16
         d_rows, d_cnt = DeviceArray((H, cap), np.int32), DeviceArray((H,), np.int32)
@@ -124,14 +131,16 @@ def _check_layer_at_size(dtype, B, N, H, Mc, density, seed):
         _capi.check(fn("sb_compute_activation_rows")(d_act2.ptr, d_xs.ptr, d_w.ptr, d_bias.ptr, d_rows.ptr,
                                                      d_cnt.ptr, cap, B, N, H, Mc, None))
         assert np.array_equal(d_cnt.numpy(), np.count_nonzero(wmask, axis=0))
-        assert np.max(np.abs(d_act2.numpy() - act)) <= 16 * tol
+        record_error("rows vs dense", np.max(np.abs(d_act2.numpy() - act)), tol)
+        assert np.max(np.abs(d_act2.numpy() - act)) <= tol
         # ... and the same from the inputs laid out in blocks of 16 rows
         d_xb = DeviceArray(((B + 15) // 16 * 16 * N,), dtype)
         _capi.check(fn("sb_rows_in_blocks")(d_xb.ptr, d_xs.ptr, B, N))
         _capi.check(lib.sb_fill_bytes(d_act2.ptr, 0, B * M * es))
         _capi.check(fn("sb_compute_activation_rows")(d_act2.ptr, d_xs.ptr, d_w.ptr, d_bias.ptr, d_rows.ptr,
                                                      d_cnt.ptr, cap, B, N, H, Mc, d_xb.ptr))
-        assert np.max(np.abs(d_act2.numpy() - act)) <= 16 * tol
+        record_error("blocked rows vs dense", np.max(np.abs(d_act2.numpy() - act)), tol)
+        assert np.max(np.abs(d_act2.numpy() - act)) <= tol
 
 
 def test_more_than_2_31_synapses_f32():

@@ -30,15 +30,15 @@ def test_reference_trajectory_fixture_f64(hb):
     net.fit(g["X"], g["Y"], int(c["B"]), [(0, int(c["l1_epochs"]))])
     assert np.array_equal(l0.wmask, g["mid_L0_wmask"])
     for name in ("weights", "bias", "Ci", "Cj", "Cij", "kbi"):
-        assert rel_err(getattr(l0, name), g[f"mid_L0_{name}"]) <= 1e-11, name
+        assert rel_err(getattr(l0, name), g[f"mid_L0_{name}"], f"mid_L0.{name}", 1e-12) <= 1e-12, name
     net.fit(g["X"], g["Y"], int(c["B"]), [(1, int(c["l2_epochs"]))])
     for li, layer in enumerate((l0, l1)):
         for name in ("weights", "bias", "Ci", "Cj", "Cij"):
-            assert rel_err(getattr(layer, name), g[f"final_L{li}_{name}"]) <= 1e-11, f"L{li}.{name}"
+            assert rel_err(getattr(layer, name), g[f"final_L{li}_{name}"], f"final_L{li}.{name}", 1e-12) <= 1e-12, f"L{li}.{name}"
     correct, total = net.evaluate(g["Xt"], g["Yt"], int(c["B"]))
     assert correct.tolist() == g["correct"].tolist() and total.tolist() == g["total"].tolist()
     assert np.array_equal(net.predict(g["Xt"], int(c["B"])), g["test_predictions"])
-    assert rel_err(net.forward(g["Xt"], int(c["B"])), g["test_activations"]) <= 1e-11
+    assert rel_err(net.forward(g["Xt"], int(c["B"])), g["test_activations"], "test_activations", 1e-12) <= 1e-12
     np.testing.assert_array_equal(np.random.rand(4), g["rng_probe_after"])
 
 
@@ -63,15 +63,47 @@ def test_single_step_matches_cpu_backend(hb, dtype, tol):
                           hp=MNIST_HP, data_seed=7)
     for li in range(2):
         for name in ("Ci", "Cj", "Cij", "weights", "bias") + (("kbi",) if li == 0 else ()):
-            e = rel_err(getattr(g._layers[li], name), getattr(r._layers[li], name))
-            assert e <= 4 * tol, f"L{li}.{name}: {e:.3e}"
+            e = rel_err(getattr(g._layers[li], name), getattr(r._layers[li], name), f"L{li}.{name}", tol)
+            assert e <= tol, f"L{li}.{name}: {e:.3e}"
     assert np.array_equal(g._layers[0].wmask, r._layers[0].wmask)
+
+
+@pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-5), (np.float64, 1e-12)])
+def test_one_step_error_table_at_the_headline_shape(hb, dtype, tol):
+    """One training step of each layer at exactly the headline configuration's shape (batch 128,
+    1568 -> 30 x 100 -> 10, mask density 0.1) against the cpu-backend restatement: the maximum of
+    |gpu - ref| / max(|ref|, 1) per quantity is asserted against the stated tolerance and written to
+    parity_one_step_<dtype>.md in $SB_PARITY_OUT (when set), the table the design notes carry."""
+    (g, r), _ = _run_both(hb, dtype, n_pix=784, H=30, Mc=100, n_out=10, Ns=128, Nt=8, B=128, e1=1, e2=1,
+                          hp=MNIST_HP, data_seed=1001)
+    rng = np.random.default_rng(1001)
+    X = synthetic_images(rng, 128, 784).astype(dtype)  # the training batch again (same generator state)
+    rows = []
+    for li in range(2):
+        for name in ("Ci", "Cj", "Cij", "weights", "bias") + (("kbi",) if li == 0 else ()):
+            e = rel_err(getattr(g._layers[li], name), getattr(r._layers[li], name), f"L{li}.{name}", tol)
+            rows.append((f"layer {li} {name}", e))
+    act_r = [r._layers[0].compute_activation(X)]
+    act_r.append(r._layers[1].compute_activation(act_r[0]))
+    for li in range(2):
+        e = rel_err(g.forward(X, 128, last_layer=li), act_r[li], f"L{li}.activations", tol)
+        rows.append((f"layer {li} activations (after the step)", e))
+    assert np.array_equal(g._layers[0].wmask, r._layers[0].wmask)
+    assert np.array_equal(g.predict(X, 128), r.predict(X, 128))
+    out = os.environ.get("SB_PARITY_OUT")
+    if out and os.path.isdir(out):
+        with open(os.path.join(out, f"parity_one_step_{np.dtype(dtype).name}.md"), "w") as f:
+            f.write(f"| quantity ({np.dtype(dtype).name}, tolerance {tol:.0e}) | max error |\n|---|---|\n")
+            for what, e in rows:
+                f.write(f"| {what} | {e:.2e} |\n")
+    for what, e in rows:
+        assert e <= tol, f"{what}: {e:.3e} > {tol:.0e}"
 
 
 def _compare_states(g, r, tol, names=("Ci", "Cj", "Cij", "weights", "bias")):
     for li in range(2):
         for name in names:
-            e = rel_err(getattr(g._layers[li], name), getattr(r._layers[li], name))
+            e = rel_err(getattr(g._layers[li], name), getattr(r._layers[li], name), f"L{li}.{name}", tol)
             assert e <= tol, f"L{li}.{name}: {e:.3e} > {tol:.1e}"
 
 
@@ -87,7 +119,7 @@ def test_small_network_epochs_with_rewiring_f64(hb, B):
     (g, r), (Xt, Yt) = _run_both(hb, np.float64, n_pix=60, H=4, Mc=10, n_out=5, Ns=200, Nt=50, B=B,
                                  e1=3, e2=2, hp=dict(MNIST_HP, l1_density=0.3), data_seed=11)
     assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
-    _compare_states(g, r, 1e-10)
+    _compare_states(g, r, 1e-12)
     assert np.array_equal(g.predict(Xt, 16), r.predict(Xt, 16))
     cg, tg = g.evaluate(Xt, Yt, 16)
     cr, tr = r.evaluate(Xt, Yt, 16)
@@ -106,9 +138,9 @@ def test_odd_shaped_networks_f64(hb, n_pix, H, Mc, n_out, Ns, B, density):
     (g, r), (Xt, Yt) = _run_both(hb, np.float64, n_pix=n_pix, H=H, Mc=Mc, n_out=n_out, Ns=Ns, Nt=40, B=B,
                                  e1=3, e2=2, hp=dict(MNIST_HP, l1_density=density), data_seed=100 + n_pix)
     assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
-    _compare_states(g, r, 1e-10)
+    _compare_states(g, r, 1e-12)
     assert np.array_equal(g.predict(Xt, B), r.predict(Xt, B))
-    assert rel_err(g.forward(Xt, 7), r.forward(Xt.astype(np.float64))) <= 1e-10
+    assert rel_err(g.forward(Xt, 7), r.forward(Xt.astype(np.float64))) <= 1e-12
 
 
 def test_classifier_epochs_follow_changes_below_them_f64(hb):
@@ -136,27 +168,27 @@ def test_classifier_epochs_follow_changes_below_them_f64(hb):
         nets.append(net)
     g, r = nets
     assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
-    _compare_states(g, r, 1e-10)
+    _compare_states(g, r, 1e-12)
     assert np.array_equal(g.predict(Xt, B), r.predict(Xt, B))
 
 
 def test_small_network_one_epoch_f32(hb):
     # float32, one epoch per layer (13 batches, short last one).  Stated drift bound after one epoch:
-    # 1e-4 relative (rounding differences of ~1e-7 per step, amplified by the log of small traces).
+    # 1e-5 relative (rounding differences of ~1e-7 per step, amplified by the log of small traces).
     (g, r), (Xt, Yt) = _run_both(hb, np.float32, n_pix=60, H=4, Mc=10, n_out=5, Ns=200, Nt=50, B=16,
                                  e1=1, e2=1, hp=dict(MNIST_HP, l1_density=0.3), data_seed=11)
     assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
-    _compare_states(g, r, 1e-4)
+    _compare_states(g, r, 1e-5)
     assert np.array_equal(g.predict(Xt, 16), r.predict(Xt, 16))
 
 
 def test_mnist_shape_one_epoch_f32(hb):
     # MNIST shape (1568 -> 30x100 -> 10), float32, batch 128, 31 batches (short last one), one epoch
-    # per layer.  Stated drift bound after one epoch: 1e-4 relative; predicted labels bit-exact.
+    # per layer.  Stated drift bound after one epoch: 1e-5 relative; predicted labels bit-exact.
     (g, r), (Xt, Yt) = _run_both(hb, np.float32, n_pix=784, H=30, Mc=100, n_out=10, Ns=31 * 128 - 32,
                                  Nt=256, B=128, e1=1, e2=1, hp=MNIST_HP, data_seed=1001)
     assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
-    _compare_states(g, r, 1e-4)
+    _compare_states(g, r, 1e-5)
     assert np.array_equal(g.predict(Xt, 128), r.predict(Xt, 128))
     cg, _ = g.evaluate(Xt, Yt, 128)
     cr, _ = r.evaluate(Xt, Yt, 128)
@@ -179,8 +211,36 @@ def test_dense_hidden_layer_one_epoch_f32(hb):
     g, r = nets
     assert g._layers[0].wmask.all() and r._layers[0].wmask.all()
     for name in ("Ci", "Cj", "Cij", "weights", "bias", "kbi"):
-        e = rel_err(getattr(g._layers[0], name), getattr(r._layers[0], name))
-        assert e <= 1e-4, f"{name}: {e:.3e}"
+        e = rel_err(getattr(g._layers[0], name), getattr(r._layers[0], name), name, 1e-5)
+        assert e <= 1e-5, f"{name}: {e:.3e}"
+
+
+def test_full_epoch_drift_f32(hb, oracle_fast):
+    """The drift bound after one epoch at the headline configuration's full size: 60000 samples, 469 steps
+    of the hidden layer (1568 -> 30 x 100, mask density 0.1, batch 128, short last batch; epoch 0, so no
+    rewiring) against the cpu-backend restatement on the reference's own build flags (OpenMP,
+    -ffast-math).  Stated drift bound after a full epoch: 5e-5 relative for every trace, the weights and
+    the bias (measured: weights 9.4e-6, bias 2.8e-6, kbi 2.2e-6, Ci 8.3e-7, Cij 1.2e-7, Cj 8.2e-8 -- the
+    two builds of the restatement themselves differ by as much, since -ffast-math reorders its sums)."""
+    from oracle import cpu_backend as ob
+    rng = np.random.default_rng(1001)
+    X = synthetic_images(rng, 60000, 784).astype(np.float32)
+    nets = []
+    for backend, kw in ((hb, {}), (ob, {"oracle": oracle_fast})):
+        np.random.seed(0)
+        net = backend.Network(np.float32)
+        hp = MNIST_HP
+        net.add_layer(backend.StructuralPlasticityLayer(
+            1568, 30, 100, hp["l1_taupdt"], hp["l1_khalf"], hp["l1_pmin"], hp["l1_taubdt"], hp["l1_density"],
+            int(hp["l1_mask_iterations"]), (1, 1 / 100, 1 / 100), **kw))
+        net.add_layer(backend.DenseLayer(3000, 1, 10, hp["l2_taupdt"], (1 / 100, 1 / 10, 1 / 1000), **kw))
+        net.fit(X, np.zeros((60000, 10), np.float32), 128, [(0, 1)])
+        nets.append(net)
+    g, r = nets
+    assert np.array_equal(g._layers[0].wmask, r._layers[0].wmask)
+    for name in ("Ci", "Cj", "Cij", "weights", "bias", "kbi"):
+        e = rel_err(getattr(g._layers[0], name), getattr(r._layers[0], name), name, 5e-5)
+        assert e <= 5e-5, f"{name}: {e:.3e}"
 
 
 def test_wide_hidden_layer_f64(hb):
@@ -189,7 +249,7 @@ def test_wide_hidden_layer_f64(hb):
     (g, r), (Xt, Yt) = _run_both(hb, np.float64, n_pix=784, H=100, Mc=100, n_out=10, Ns=512 + 96, Nt=64,
                                  B=512, e1=1, e2=1, hp=MNIST_HP, data_seed=1002)
     assert _mask_diff(g._layers[0].wmask, r._layers[0].wmask) == 0
-    _compare_states(g, r, 1e-11)
+    _compare_states(g, r, 1e-12)
     assert np.array_equal(g.predict(Xt, 512), r.predict(Xt, 512))
 
 
@@ -329,25 +389,25 @@ def test_forward_over_connected_rows_tracks_the_state(hb, dtype, tol):
         return k.compute_activation(np.ascontiguousarray(W), np.ascontiguousarray(b), xt, 6, 20)
 
     # before any training step W is the unmasked initial draw: dense path
-    assert rel_err(net.forward(xt, last_layer=0), dense(layer.weights, layer.bias)) <= 4 * tol
+    assert rel_err(net.forward(xt, last_layer=0), dense(layer.weights, layer.bias)) <= tol
     net.fit(X, Y, 64, [(0, 2)])  # two epochs, the second with rewiring
     W, b, mask = layer.weights, layer.bias, layer.wmask
     assert np.all(W[np.repeat(mask, 20, axis=1) == 0] == 0)
-    assert rel_err(net.forward(xt, last_layer=0), dense(W, b)) <= 4 * tol  # row lists (after rewiring)
+    assert rel_err(net.forward(xt, last_layer=0), dense(W, b)) <= tol  # row lists (after rewiring)
     # a masked W written from outside (a restored checkpoint) is recognised as such ...
     layer.weights = W
-    assert rel_err(net.forward(xt, last_layer=0), dense(W, b)) <= 4 * tol
+    assert rel_err(net.forward(xt, last_layer=0), dense(W, b)) <= tol
     # ... and an unmasked one must be used as it is
     W2 = (W + 0.01).astype(dtype)
     layer.weights = W2
-    assert rel_err(net.forward(xt, last_layer=0), dense(W2, b)) <= 4 * tol
+    assert rel_err(net.forward(xt, last_layer=0), dense(W2, b)) <= tol
     # ... and a new mask does not touch W until the next training step
     layer.wmask = np.ascontiguousarray(1 - mask)
-    assert rel_err(net.forward(xt, last_layer=0), dense(W2, b)) <= 4 * tol
+    assert rel_err(net.forward(xt, last_layer=0), dense(W2, b)) <= tol
     net.fit(X, Y, 64, [(0, 1)])
     W3, mask3 = layer.weights, layer.wmask
     assert np.all(W3[np.repeat(mask3, 20, axis=1) == 0] == 0)
-    assert rel_err(net.forward(xt, last_layer=0), dense(W3, layer.bias)) <= 4 * tol
+    assert rel_err(net.forward(xt, last_layer=0), dense(W3, layer.bias)) <= tol
 
 
 def test_full_size_epochs_keep_the_invariants_f32(hb):
