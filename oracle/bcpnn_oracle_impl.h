@@ -148,11 +148,16 @@ void FN(oracle_update_bias_regularized)(REAL *bias, REAL *kbi, const REAL *Cj, R
 /* omp.cc:248-320 (update_mask).  The score quotient is evaluated in double and narrowed, because the
  * reference writes nominator / (1.0 + (REAL)csum) (omp.cc:293).  Candidates are scanned in ascending
  * row order with >= / <=, so among equal scores the LAST row wins (omp.cc:294-304).
- * Optional trace output (may be NULL): per executed swap, swaps[4*t..] = {imax0, imin1} and
- * vals[2*t..] = {vmax0, vmin1}; *nswaps receives the number of swaps performed. */
+ * Optional trace output (each may be NULL): per executed swap, swaps[2*t..] = {imax0, imin1},
+ * vals[2*t..] = {vmax0, vmin1} and runner[2*t..] = {the best score among the other silent rows, the worst
+ * among the other active rows} at that iteration (the margins by which the two picks won; -3e38 / +3e38
+ * when a side had one candidate only); *nswaps receives the number of swaps performed; stop[0..2] =
+ * {1, vmax0, vmin1} when the loop ended by vmax0 < vmin1, {0, 0, 0} otherwise.  The trace changes nothing of
+ * the result. */
 void FN(oracle_update_mask)(uint8_t *wmask, const REAL *W, const REAL *Ci, const REAL *Cj,
                             const REAL *Cij, REAL cthr, long N, long M, long h, long H, long Mc,
-                            long iterations, long *swaps, REAL *vals, long *nswaps) {
+                            long iterations, long *swaps, REAL *vals, long *nswaps, REAL *runner,
+                            REAL *stop) {
   REAL *nom = (REAL *)calloc((size_t)N, sizeof(REAL));
   int *csum = (int *)calloc((size_t)N, sizeof(int));
 #pragma omp parallel for schedule(static)
@@ -188,7 +193,22 @@ void FN(oracle_update_mask)(uint8_t *wmask, const REAL *W, const REAL *Ci, const
         vmin1 = score;
       }
     }
+    if (stop) {
+      stop[0] = stop[1] = stop[2] = (REAL)0;
+      if (imax0 != N && imin1 != N && vmax0 < vmin1) stop[0] = (REAL)1, stop[1] = vmax0, stop[2] = vmin1;
+    }
     if (imax0 == N || imin1 == N || vmax0 < vmin1) break;
+    if (runner) { /* second scan, trace only: the runners-up of this iteration */
+      REAL r0 = (REAL)-3e38, r1 = (REAL)3e38;
+      for (long j = 0; j < N; j++) {
+        if (j == imax0 || j == imin1) continue;
+        const REAL score = (REAL)((double)nom[j] / (1.0 + (double)(REAL)csum[j]));
+        if (wmask[j * H + h] == 0 && score > r0) r0 = score;
+        else if (wmask[j * H + h] == 1 && score < r1) r1 = score;
+      }
+      runner[2 * done] = r0;
+      runner[2 * done + 1] = r1;
+    }
     wmask[imax0 * H + h] = 1;
     wmask[imin1 * H + h] = 0;
     csum[imax0] += 1;

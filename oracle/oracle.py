@@ -37,7 +37,7 @@ def load(fast=False):
             f = getattr(lib, "oracle_update_bias_regularized" + sfx)
             f.argtypes = [_P, _P, _P, R, R, R, R, _L]; f.restype = None
             f = getattr(lib, "oracle_update_mask" + sfx)
-            f.argtypes = [_P, _P, _P, _P, _P, R, _L, _L, _L, _L, _L, _L, _P, _P, _P]; f.restype = None
+            f.argtypes = [_P, _P, _P, _P, _P, R, _L, _L, _L, _L, _L, _L, _P, _P, _P, _P, _P]; f.restype = None
             f = getattr(lib, "oracle_apply_mask" + sfx)
             f.argtypes = [_P, _P, _L, _L, _L, _L]; f.restype = None
             f = getattr(lib, "oracle_argmax_rows" + sfx)
@@ -126,10 +126,12 @@ class Oracle:
         N, M = weights.shape
         assert wmask.shape == (N, hypercolumns) and wmask.dtype == np.uint8
         assert M == hypercolumns * minicolumns and 0 <= h < hypercolumns
-        swaps = vals = nsw = None
+        swaps = vals = nsw = runner = stop = None
         if trace is not None:
             swaps = np.zeros([max(iterations, 1), 2], dtype=np.int64)
             vals = np.zeros([max(iterations, 1), 2], dtype=d)
+            runner = np.zeros([max(iterations, 1), 2], dtype=d)
+            stop = np.zeros([3], dtype=d)
             nsw = ctypes.c_long(0)
         getattr(self.lib, "oracle_update_mask" + s)(
             _chk(wmask, np.uint8, "wmask"), _chk(weights, d, "weights"), _chk(Ci, d, "Ci"),
@@ -137,10 +139,16 @@ class Oracle:
             iterations,
             swaps.ctypes.data if swaps is not None else None,
             vals.ctypes.data if vals is not None else None,
-            ctypes.byref(nsw) if nsw is not None else None)
+            ctypes.byref(nsw) if nsw is not None else None,
+            runner.ctypes.data if runner is not None else None,
+            stop.ctypes.data if stop is not None else None)
         if trace is not None:
+            # per swap: the rows picked, their scores, the runners-up on either side (-3e38 / 3e38: none);
+            # stop: (vmax0, vmin1) of the iteration that ended the loop by vmax0 < vmin1, or None
             trace["swaps"] = swaps[:nsw.value].copy()
             trace["vals"] = vals[:nsw.value].copy()
+            trace["runner"] = runner[:nsw.value].copy()
+            trace["stop"] = (float(stop[1]), float(stop[2])) if stop[0] != 0 else None
         return wmask
 
     # kernels_openmp.py:90-99

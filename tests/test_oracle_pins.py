@@ -301,6 +301,45 @@ def test_update_mask_vs_brute_force(oracle, seed):
         assert (got != wmask).sum() <= 2 * iterations
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_update_mask_trace_vs_brute_force(oracle, seed):
+    """The optional trace of the rewiring (rows picked, their scores, the runners-up on either side, the
+    scores that ended the loop) against a Python scan in float64 on float64 inputs."""
+    rng = np.random.default_rng(300 + seed)
+    N, H, Mc = int(rng.integers(6, 40)), int(rng.integers(1, 5)), int(rng.integers(2, 7))
+    wmask, W, Ci, Cj, Cij = _mask_problem(rng, N, H, Mc)
+    h = int(rng.integers(0, H))
+    trace = {}
+    oracle.update_mask(wmask.copy(), W, Ci, Cj, Cij, 0.01, H, Mc, h, 16, trace=trace)
+    wm = wmask.copy().astype(int)
+    nom = np.zeros(N)
+    for i in range(N):
+        for j in range(h * Mc, (h + 1) * Mc):
+            if Ci[i] >= 0.01 and Cj[j] >= 0.01:
+                nom[i] += Cij[i, j] * W[i, j] + (Cj[j] - Cij[i, j]) * np.log((Cj[j] - Cij[i, j]) / ((1 - Ci[i]) * Cj[j]))
+    swaps, stop = [], None
+    for _ in range(16):
+        score = nom / (1.0 + wm.sum(1))
+        zeros, ones = np.flatnonzero(wm[:, h] == 0), np.flatnonzero(wm[:, h] == 1)
+        if not len(zeros) or not len(ones):
+            break
+        imax = max(i for i in zeros if score[i] == score[zeros].max())
+        imin = max(i for i in ones if score[i] == score[ones].min())
+        if score[imax] < score[imin]:
+            stop = (score[imax], score[imin])
+            break
+        r0 = max((score[i] for i in zeros if i != imax), default=-3e38)
+        r1 = min((score[i] for i in ones if i != imin), default=3e38)
+        swaps.append((imax, imin, score[imax], score[imin], r0, r1))
+        wm[imax, h], wm[imin, h] = 1, 0
+    assert trace["swaps"].tolist() == [[a, b] for a, b, *_ in swaps]
+    assert np.allclose(trace["vals"], [[c, d] for _, _, c, d, _, _ in swaps] or np.zeros((0, 2)), rtol=1e-12, atol=0)
+    assert np.allclose(trace["runner"], [[e, f] for *_, e, f in swaps] or np.zeros((0, 2)), rtol=1e-12, atol=0)
+    assert (trace["stop"] is None) == (stop is None)
+    if stop is not None:
+        assert np.allclose(trace["stop"], stop, rtol=1e-12, atol=0)
+
+
 def test_update_mask_degenerate_columns_and_ties(oracle):
     rng = np.random.default_rng(4)
     N, H, Mc = 10, 2, 3
