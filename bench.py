@@ -1,23 +1,30 @@
 #!/usr/bin/env python3
 """Benchmark of the BCPNN layer training step on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
-  python bench.py --workload dense|mnist15x200|wide64|stl10|largest    (other configurations, see LARGE below)
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-other-configs]
+  python bench.py --workload dense|mnist15x200|wide64|stl10|largest    one of the other configurations alone
+  python bench.py --achievable-peaks                                   device-copy and matrix-core probes
+  python bench.py --copy-calibration                                   known-size copies for counter scaling
+  python bench.py --pmc-summary DIR                                    text summary of rocprofv3 --pmc runs
 
-Workload: the MNIST-shaped 2-layer network, float32, batch 128, 60000 seeded
+Headline workload: the MNIST-shaped 2-layer network, float32, batch 128, 60000 seeded
 synthetic samples; input 784 pixels complementary-coded to 1568 units (~19% nonzero pixels, uniform
 in (0,1]); hidden layer 30 hypercolumns x 100 minicolumns with a receptive-field mask of density 0.1;
 10-class dense output layer.  A "step" is one structural-plasticity-layer training step on one
 resident batch: forward x.W+b with per-hypercolumn softmax, Ci/Cj/Cij trace update, weight and bias
 recompute, mask apply, and the mask rewiring at the reference's cadence (every 15th step of an epoch
-after the first).  The timed region starts with the training set already in HBM.
+after the first).  The timed region starts with the training set already in HBM.  The window of K steps
+is timed several times; `value` and `ms_per_step` are the median window, `windows` holds the spread.
 
 Prints one JSON line.  `value` is training samples/s; `roofline` describes the dominant kernel (the
-fused trace+weight pass); `cpu_baseline` is the CPU oracle (the reference's OpenMP loop structure,
-built with the reference's flag set) timed on this host on a bounded number of the same steps.
+fused trace+weight pass); `cpu_baseline` is the CPU restatement of the reference's cpu backend (its
+OpenMP loop structure built with its flag set, the forward product through numpy's BLAS, numpy softmax)
+timed on this host on a bounded number of the same steps, with a per-function split; `other_configs`
+holds short runs of the other four configurations, each with its own roofline and CPU baseline.
 """
 import argparse
 import ctypes
+import hashlib
 import json
 import os
 import sys
@@ -32,6 +39,9 @@ N_PIXELS, H, MC, N_OUT, BATCH, N_SAMPLES = 784, 30, 100, 10, 128, 60000
 HP = dict(l1_taupdt=0.006908854922437549, l1_pmin=0.06195283356566607, l1_khalf=-139.02586632856327,
           l1_taubdt=0.02218100432360414, l1_density=0.1, l2_taupdt=0.0007449780036161324)
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}
+PMC_PROFILE = os.path.join(ROOT, "profiles", "k_train_fused_mnist_f32_b128_pmc.txt")
+KERNEL_SOURCES = ("sb_k_train.hpp", "sb_common.hpp")
 
 
 def synthetic_dataset(n, seed=1001):
@@ -74,6 +84,136 @@ def batch_plan(first_step, n_steps, nb):
     return out
 
 
+def window_stats(times_s, samples, steps):
+    """Median window (the reported one) and the spread over the timed windows of `steps` steps each."""
+    order = np.argsort(times_s)
+    mid = int(order[len(order) // 2])
+    per_step = [1e3 * t / steps for t in times_s]
+    return mid, {"count": len(times_s), "steps_each": steps, "ms_per_step_median": per_step[mid],
+                 "ms_per_step_min": min(per_step), "ms_per_step_max": max(per_step)}
+
+
+def n_windows(steps):
+    """How often the window of `steps` steps is timed: about 3000 steps in all, 3 to 50 windows."""
+    return int(min(50, max(3, -(-3000 // max(steps, 1)))))
+
+
+def host_info():
+    """CPU model, physical cores of the host and the threads the CPU baseline uses."""
+    model, cores = "unknown", set()
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name") and model == "unknown":
+                model = line.split(":", 1)[1].strip()
+            elif line.startswith("physical id"):
+                phys = line.split(":", 1)[1].strip()
+            elif line.startswith("core id"):
+                core = line.split(":", 1)[1].strip()
+            elif not line.strip():
+                if phys is not None and core is not None:
+                    cores.add((phys, core))
+                phys = core = None
+    except OSError:
+        pass
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    blas = "unknown"
+    try:
+        cfg = np.show_config(mode="dicts")
+        b = cfg.get("Build Dependencies", {}).get("blas", {})
+        blas = f"{b.get('name', 'unknown')} {b.get('version', '')}".strip()
+    except Exception:
+        pass
+    return {"cpu_model": model, "physical_cores_of_host": len(cores) or None, "logical_cpus_of_host": os.cpu_count(),
+            "threads_used": threads, "numpy_blas": blas}
+
+
+# ---------------------------------------------------------------------------------------- CPU baseline
+def numpy_softmax(a, h, mc):
+    """kernels_numpy.py:13-25 of the reference (what its cpu backend binds for the softmax)."""
+    t = a.reshape(-1, h, mc)
+    t = np.exp(t - t.max(axis=2, keepdims=True))
+    return (t / t.sum(axis=2, keepdims=True)).reshape(a.shape)
+
+
+def cpu_baseline(x, st, h, mc, batch, tau, dtype, budget_s, min_steps=1, rewire_period=15, warm=True):
+    """The cpu backend's training step of one structural-plasticity layer on this host: forward product
+    through numpy's BLAS (the reference calls cblas), numpy softmax (the reference's own), and the C
+    restatement of its OpenMP kernels built with its flag set for the fused trace + weight pass, the
+    regularised bias, the rewiring and the mask apply.  Batches in storage order, a rewiring every
+    `rewire_period`-th step; at least min_steps timed steps, then until budget_s is used up."""
+    from concurrent.futures import ThreadPoolExecutor
+    from threadpoolctl import threadpool_limits
+    from oracle.oracle import Oracle
+    o = Oracle(fast=True)
+    cthr = tau / 2
+    info = host_info()
+    full_batches = max(1, x.shape[0] // batch)
+    split = {"forward_blas": 0.0, "softmax_numpy": 0.0, "traces_and_weights": 0.0, "bias": 0.0, "mask": 0.0}
+    # The forward product runs numpy's BLAS kernel on every core, one column slice of W per thread with the
+    # library's own threading off: its worker threads would otherwise keep spinning after each product
+    # and take the cores from the OpenMP loops that follow (measured: those loops ran 2.4 times slower).
+    threads = info["threads_used"]
+    m = st["weights"].shape[1]
+    cuts = [m * k // threads for k in range(threads + 1)]
+    pool = ThreadPoolExecutor(threads)
+    limit = threadpool_limits(limits=1, user_api="blas")
+
+    def forward(xb):
+        act = np.empty((xb.shape[0], m), dtype=dtype)
+
+        def part(k):
+            np.matmul(xb, st["weights"][:, cuts[k]:cuts[k + 1]], out=act[:, cuts[k]:cuts[k + 1]])
+        list(pool.map(part, range(threads)))
+        act += st["bias"]
+        return act
+
+    def step(i, timed):
+        i = i % full_batches
+        xb = x[i * batch:(i + 1) * batch]
+        t = [time.perf_counter()]
+        act = forward(xb)
+        t.append(time.perf_counter())
+        act = np.ascontiguousarray(numpy_softmax(act, h, mc), dtype=dtype)
+        t.append(time.perf_counter())
+        o.update_weights(st["Ci"], st["Cj"], st["Cij"], xb, act, tau, st["weights"], cthr)
+        t.append(time.perf_counter())
+        o.update_bias_regularized(st["bias"], st["kbi"], st["Cj"], cthr, HP["l1_khalf"], HP["l1_pmin"],
+                                  HP["l1_taubdt"])
+        t.append(time.perf_counter())
+        if rewire_period and i % rewire_period == 0 and i // rewire_period < h:
+            o.update_mask(st["wmask"], st["weights"], st["Ci"], st["Cj"], st["Cij"], cthr, h, mc,
+                          i // rewire_period, 16)
+        o.apply_mask(st["weights"], st["wmask"], h, mc)
+        t.append(time.perf_counter())
+        if timed:
+            for name, a, b in zip(split, t[:-1], t[1:]):
+                split[name] += b - a
+        return xb.shape[0]
+
+    if warm:
+        step(0, False)  # thread pool, page faults
+    t0 = time.perf_counter()
+    samples = steps = 0
+    while steps < min_steps or time.perf_counter() - t0 < budget_s:
+        samples += step(1 + steps, True)
+        steps += 1
+        if steps >= 100000:
+            break
+    dt = time.perf_counter() - t0
+    pool.shutdown()
+    limit.restore_original_limits()
+    return {"value": samples / dt, "unit": "samples/s", "cores": info["threads_used"], "kind": "port",
+            "sample": f"{steps} training step(s) of the same workload (batch {batch}"
+                      + (f", rewiring every {rewire_period}th step" if rewire_period else ", no rewiring")
+                      + f"), {dt:.1f} s" + ("" if warm else ", no warm-up step")
+                      + "; C restatement built -O3 -march=x86-64-v3 -ffast-math -fopenmp, forward through numpy's BLAS kernel, one column slice of W per thread",
+            "ms_per_step": 1e3 * dt / max(steps, 1),
+            "ms_per_step_by_function": {k: 1e3 * v / max(steps, 1) for k, v in split.items()},
+            "host": info}
+
+
+# ------------------------------------------------------------------------------------------- headline
 class DeviceRun:
     def __init__(self, x, y):
         from streambrain_amd import _capi
@@ -97,6 +237,10 @@ class DeviceRun:
         self.ns = x.shape[0]
         self.nb = (self.ns + BATCH - 1) // BATCH
         self.rng = np.random.default_rng(7)
+
+    def close(self):
+        self.capi.check(self.lib.sb_net_destroy(self.net))
+        self.net = None
 
     def run_steps(self, first_step, n_steps):
         """Enqueues steps [first_step, first_step + n_steps); returns the number of samples."""
@@ -140,244 +284,52 @@ class DeviceRun:
         self.capi.check(self.lib.sb_profile_start())
         self.run_steps(first_step, n_steps)
         self.capi.check(self.lib.sb_profile_stop())
-        out = {}
-        self.raw_bracket_ms, self.brackets = 0.0, 0
-        for k in range(self.lib.sb_profile_kernels()):
-            ms, n = ctypes.c_double(0), ctypes.c_long(0)
-            self.capi.check(self.lib.sb_profile_get(k, ctypes.byref(ms), ctypes.byref(n)))
-            self.raw_bracket_ms += ms.value
-            self.brackets += n.value
-            if n.value:
-                out[self.lib.sb_profile_kernel_name(k).decode()] = {
-                    "launches": n.value, "avg_us": 1e3 * ms.value / n.value}
-        return out
+        return read_profile(self.lib, self.capi.check)
 
 
-def cpu_baseline(x, y, budget_s=15.0, max_steps=100000):
-    """The CPU oracle (reference loop structure, reference flag set, OpenMP) on the first steps of the
-    same workload: same initial state, same data, batches in storage order, rewiring every 15th step."""
-    from oracle.oracle import Oracle
-    o = Oracle(fast=True)
-    st = initial_state()
-    tau, cthr = HP["l1_taupdt"], HP["l1_taupdt"] / 2
-    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-
-    full_batches = x.shape[0] // BATCH
-
-    def step(i):
-        i = i % full_batches
-        xb = x[i * BATCH:(i + 1) * BATCH]
-        act = np.zeros((xb.shape[0], H * MC), dtype=np.float32)
-        o.update_state(act, st["weights"], st["bias"], xb)
-        o.softmax_minicolumns(act, H, MC)
-        o.update_weights(st["Ci"], st["Cj"], st["Cij"], xb, act, tau, st["weights"], cthr)
-        o.update_bias_regularized(st["bias"], st["kbi"], st["Cj"], cthr, HP["l1_khalf"], HP["l1_pmin"],
-                                  HP["l1_taubdt"])
-        if i % 15 == 0 and i // 15 < H:
-            o.update_mask(st["wmask"], st["weights"], st["Ci"], st["Cj"], st["Cij"], cthr, H, MC, i // 15, 16)
-        o.apply_mask(st["weights"], st["wmask"], H, MC)
-        return xb.shape[0]
-
-    step(0)  # warm-up (thread pool, page faults)
-    t0 = time.perf_counter()
-    samples = steps = 0
-    while steps < max_steps and time.perf_counter() - t0 < budget_s:
-        samples += step(1 + steps)
-        steps += 1
-    dt = time.perf_counter() - t0
-    return {"value": samples / dt, "unit": "samples/s", "cores": threads, "kind": "port",
-            "sample": f"{steps} training steps of the same workload (batch {BATCH}, rewiring every 15th step), "
-                      f"{dt:.1f} s, oracle built -O3 -march=x86-64-v3 -ffast-math -fopenmp",
-            "ms_per_step": 1e3 * dt / max(steps, 1)}
-
-
-# Other layer shapes, run through the same network path (one structural-plasticity layer, data resident in
-# HBM, first epoch: no rewiring).  in_features, hypercolumns, minicolumns, batch, mask density, dtype,
-# samples kept on the device (an epoch of the run cycles through them), fraction of non-zero inputs.
-LARGE = {
-    "dense": dict(n=1568, h=30, mc=100, batch=128, density=1.0, dtype=np.float32, samples=60000, nonzero=0.19,
-                  what="configs[0]: single hidden layer 1568 -> 30x100, float32, batch 128, dense (no mask), one epoch"),
-    "stl10": dict(n=55296, h=200, mc=100, batch=256, density=0.05, dtype=np.float32, samples=5000, nonzero=1.0,
-                  what="configs[3]: STL-10-shaped layer 55296 -> 200x100, float32, batch 256, mask density 0.05"),
-    "largest": dict(n=65536, h=1000, mc=100, batch=1024, density=1.0, dtype=np.float32, samples=4096, nonzero=0.2,
-                    what="configs[4]: 65536 -> 1000x100, float32, batch 1024, binary inputs, dense mask"),
-    "mnist15x200": dict(n=1568, h=15, mc=200, batch=128, density=0.1, dtype=np.float32, samples=60000, nonzero=0.19,
-                        what="the reference example script's own MNIST layer: 1568 -> 15x200, float32, batch 128, "
-                             "mask density 0.1"),
-    "wide64": dict(n=1568, h=100, mc=100, batch=512, density=0.1, dtype=np.float64, samples=60000, nonzero=0.19,
-                   what="configs[2]: 1568 -> 100x100, float64, batch 512, mask density 0.1"),
-}
-
-
-def large_workload(name, steps, warmup):
-    """Training steps of one structural-plasticity layer of a LARGE shape; prints one JSON line of the same
-    form as the headline run (no CPU baseline: the oracle needs minutes per step at these sizes)."""
-    from streambrain_amd import _capi
-    cfg = LARGE[name]
-    n, h, mc, batch, dt = cfg["n"], cfg["h"], cfg["mc"], cfg["batch"], cfg["dtype"]
-    m, ns, es = h * mc, cfg["samples"], np.dtype(cfg["dtype"]).itemsize
-    rng = np.random.default_rng(1000 + len(name))
-    if name == "largest":
-        x = (rng.random((ns, n), dtype=np.float32) < cfg["nonzero"]).astype(dt)
-    else:
-        half = n // 2
-        px = rng.random((ns, half), dtype=np.float32)
-        if cfg["nonzero"] < 1.0:
-            px *= rng.random((ns, half), dtype=np.float32) < cfg["nonzero"]
-        x = np.concatenate([px, 1.0 - px], axis=1).astype(dt)
-    lib = _capi.lib()
-    _capi.init(0)
-    c = _capi.check
-    net = ctypes.c_void_p()
-    c(lib.sb_net_create(ctypes.byref(net), 0 if dt == np.float32 else 1))
-    tau = HP["l1_taupdt"] * np.sqrt(batch / 128.0)
-    c(lib.sb_net_add_plastic_layer(net, n, h, mc, tau, HP["l1_pmin"], HP["l1_khalf"], HP["l1_taubdt"], 1.0,
-                                   1.0 / mc, 1.0 / mc))
-    # a (never trained) output layer behind it, so that the layer trains on its own activation
-    c(lib.sb_net_add_dense_layer(net, m, 1, N_OUT, HP["l2_taupdt"], 1.0 / mc, 1.0 / N_OUT, 1.0 / mc / N_OUT))
-    connected = n * h
-    if cfg["density"] < 1.0:
-        wmask = (rng.random((n, h), dtype=np.float32) < cfg["density"]).astype(np.uint8)
-        connected = int(np.count_nonzero(wmask))
-        c(lib.sb_net_set_layer_state(net, 0, b"wmask", wmask.ctypes.data, wmask.nbytes))
-    c(lib.sb_net_set_training_data(net, x.ctypes.data, None, ns, n, 0))
-    nb = (ns + batch - 1) // batch
-
-    def run(first, count):
-        done = 0
-        for epoch, fb, take in batch_plan(first, count, nb):
-            perm = rng.permutation(ns).astype(np.int64) if fb == 0 else None
-            hc = rng.permutation(h).astype(np.int64)
-            c(lib.sb_net_train_batches(net, 0, batch, perm.ctypes.data if perm is not None else None,
-                                       hc.ctypes.data, 0, fb, take, 0))
-            done += sum(min(batch, ns - b * batch) for b in range(fb, fb + take))
-        return done
-
-    warmup = max(warmup, 1)
-    warmup += (-warmup) % nb  # the timed region starts at an epoch boundary
-    run(0, warmup)
-    c(lib.sb_sync())
-    t0 = time.perf_counter()
-    samples = run(warmup, steps)
-    c(lib.sb_sync())
-    dt_s = time.perf_counter() - t0
-    c(lib.sb_profile_start())
-    n_prof = min(steps, nb)
-    run(warmup + steps + (-(warmup + steps)) % nb, n_prof)
-    c(lib.sb_profile_stop())
-    kernels, raw_ms, brackets = {}, 0.0, 0
+def read_profile(lib, check):
+    """Per-kernel sums of the HIP-event brackets of the last profiled pass: ({name: {launches, raw_avg_us}},
+    summed bracket time in ms, number of brackets)."""
+    out, raw_ms, brackets = {}, 0.0, 0
     for k in range(lib.sb_profile_kernels()):
-        ms, cnt = ctypes.c_double(0), ctypes.c_long(0)
-        c(lib.sb_profile_get(k, ctypes.byref(ms), ctypes.byref(cnt)))
+        ms, n = ctypes.c_double(0), ctypes.c_long(0)
+        check(lib.sb_profile_get(k, ctypes.byref(ms), ctypes.byref(n)))
         raw_ms += ms.value
-        brackets += cnt.value
-        if cnt.value:
-            kernels[lib.sb_profile_kernel_name(k).decode()] = {"launches": cnt.value,
-                                                               "raw_avg_us": 1e3 * ms.value / cnt.value}
-    # what a HIP-event bracket adds to a launch, from the two passes (as in the headline run)
-    bracket_us = max(0.0, (1e3 * raw_ms - 1e6 * dt_s * n_prof / steps) / max(brackets, 1))
+        brackets += n.value
+        if n.value:
+            out[lib.sb_profile_kernel_name(k).decode()] = {"launches": n.value, "raw_avg_us": 1e3 * ms.value / n.value}
+    return out, raw_ms, brackets
+
+
+def calibrate_brackets(kernels, raw_ms, brackets, unbracketed_s):
+    """A HIP-event bracket adds a little to each launch; how much follows from the two passes themselves:
+    (sum of all brackets - wall time of the same steps without brackets) / brackets."""
+    bracket_us = max(0.0, (1e3 * raw_ms - 1e6 * unbracketed_s) / max(brackets, 1))
     for k in kernels.values():
         k["avg_us"] = max(k["raw_avg_us"] - bracket_us, 0.0)
-    tw = kernels.get("train_fused", {"avg_us": float("nan")})["avg_us"] * 1e-6
-    fw = kernels.get("forward", {"avg_us": float("nan")})["avg_us"] * 1e-6
-    peak = 157.3 if dt == np.float32 else 78.6
-    gemm = 2.0 * batch * n * m  # the Cij trace GEMM of a full batch; bound: MFMA at these batch sizes
-    fwd_flops = 2.0 * batch * connected * mc if cfg["density"] <= 0.5 else gemm
-    print(json.dumps({
-        "metric": "train samples/sec on 1 MI355X; % HBM / MFMA peak",
-        "value": samples / dt_s, "unit": "samples/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
-        "ms_per_step": 1e3 * dt_s / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if dt == np.float32 else "f64", "data": "synthetic",
-        "config": {"workload": cfg["what"], "batch": batch, "in_features": n, "hypercolumns": h,
-                   "minicolumns": mc, "samples": ns},
-        "roofline": {"bound": "mfma", "kernel": "k_train_fused", "achieved": gemm / tw / 1e12, "peak": peak,
-                     "unit": "TFLOP/s", "frac": gemm / tw / 1e12 / peak, "traffic": None,
-                     "algorithmic_flops_per_launch": gemm, "avg_launch_us": tw * 1e6,
-                     "bytes_3sNM_per_launch": 3 * es * n * m, "achieved_GBps_on_3sNM": 3 * es * n * m / tw / 1e9},
-        "mfma": {"kernel": "k_forward_rows" if cfg["density"] <= 0.5 else "k_forward",
-                 "flops_per_launch": fwd_flops, "achieved_tflops": fwd_flops / fw / 1e12, "peak_tflops": peak,
-                 "frac": fwd_flops / fw / 1e12 / peak, "avg_launch_us": fw * 1e6},
-        "kernels": kernels, "event_bracket_overhead_us": {"calibrated": bracket_us}, "cpu_baseline": None}))
-    return 0
+    return bracket_us
 
 
-def measured_traffic():
-    """HBM bytes per launch of the dominant kernel, as measured with rocprofv3 --pmc FETCH_SIZE /
-    WRITE_SIZE and recorded in profiles/ (line `traffic_bytes_per_launch: N`); None when absent."""
-    path = os.path.join(ROOT, "profiles", "k_train_fused_mnist_f32_b128_pmc.txt")
-    try:
-        for line in open(path):
-            if line.startswith("traffic_bytes_per_launch:"):
-                return float(line.split(":", 1)[1])
-    except OSError:
-        pass
-    return None
-
-
-def copy_calibration(nbytes=64 << 20, copies=6):
-    from streambrain_amd import _capi
-    from streambrain_amd._capi import DeviceArray
-    _capi.init(0)
-    lib = _capi.lib()
-    src, dst = DeviceArray((nbytes,), np.uint8), DeviceArray((nbytes,), np.uint8)
-    _capi.check(lib.sb_fill_bytes(src.ptr, 1, nbytes))
-    _capi.check(lib.sb_fill_bytes(dst.ptr, 2, nbytes))
-    for _ in range(copies):
-        _capi.check(lib.sb_memcpy_d2d(dst.ptr, src.ptr, nbytes))
-    _capi.check(lib.sb_sync())
-    print(json.dumps({"copy_calibration": {"copies": copies, "bytes_read_per_copy": nbytes,
-                                           "bytes_written_per_copy": nbytes}}))
-    return 0
-
-
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=938)
-    ap.add_argument("--warmup", type=int, default=60)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-baseline-seconds", type=float, default=15.0,
-                    help="length of the CPU baseline's sample")
-    ap.add_argument("--samples", type=int, default=N_SAMPLES)
-    ap.add_argument("--workload", choices=["mnist"] + sorted(LARGE), default="mnist",
-                    help="mnist (default): the headline configuration; the others: one layer of a larger "
-                         "shape (--steps defaults to two epochs of its resident samples)")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="only run six 64 MiB device-to-device copies: the known-size kernel that "
-                         "hardware counter readings (FETCH_SIZE, WRITE_SIZE) are scaled by")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
-              "(the path is not sharded across devices)", file=sys.stderr)
-        return 2
-
-    if args.copy_calibration:
-        return copy_calibration()
-    if args.workload != "mnist":
-        cfg = LARGE[args.workload]
-        nb = (cfg["samples"] + cfg["batch"] - 1) // cfg["batch"]
-        steps = args.steps if "--steps" in sys.argv else (nb if nb > 100 else 2 * nb)
-        return large_workload(args.workload, steps, args.warmup if "--warmup" in sys.argv else nb)
-
+def headline(args):
     x, y = synthetic_dataset(args.samples)
     run = DeviceRun(x, y)
-
     run.run_steps(0, args.warmup)
     run.sync()
-    t0 = time.perf_counter()
-    samples = run.run_steps(args.warmup, args.steps)
-    run.sync()
-    dt = time.perf_counter() - t0
+    times, samples_of, first = [], [], args.warmup
+    for _ in range(n_windows(args.steps)):
+        t0 = time.perf_counter()
+        samples_of.append(run.run_steps(first, args.steps))
+        run.sync()
+        times.append(time.perf_counter() - t0)
+        first += args.steps
+    mid, windows = window_stats(times, samples_of, args.steps)
+    dt, samples = times[mid], samples_of[mid]
 
-    # Per-kernel durations: every launch of a second pass over the same number of steps is bracketed by
-    # HIP events on the library's stream.  A bracket adds a little to each launch; how much is calibrated
-    # from the two passes themselves: (sum of all brackets - wall time of the unbracketed pass) / brackets.
+    # Per-kernel durations: every launch of one more pass over the same number of steps is bracketed by
+    # HIP events on the library's stream.
     n_prof = min(args.steps, 2 * run.nb)
-    prof = run.profile(args.warmup + args.steps, n_prof)
-    bracket_us = max(0.0, (1e3 * run.raw_bracket_ms - 1e6 * dt * n_prof / args.steps) / max(run.brackets, 1))
-    for k in prof.values():
-        k["raw_avg_us"] = k["avg_us"]
-        k["avg_us"] = max(k["avg_us"] - bracket_us, 0.0)
+    prof, raw_ms, brackets = run.profile(first, n_prof)
+    bracket_us = calibrate_brackets(prof, raw_ms, brackets, dt * n_prof / args.steps)
 
     # the two other phases of the reference's example run, reported beside the headline figure
     # (the first classifier epoch also computes the frozen hidden layer's activations of the whole training
@@ -409,6 +361,9 @@ def main():
     fwd = prof.get("forward", {"avg_us": float("nan")})
     fwd_flops = 2.0 * BATCH * connected
     fwd_tflops = fwd_flops / (fwd["avg_us"] * 1e-6) / 1e12
+    gemm_tflops = 2.0 * BATCH * n * m / (tw["avg_us"] * 1e-6) / 1e12
+    traffic, traffic_note = measured_traffic()
+    run.close()
 
     result = {
         "metric": "train samples/sec on 1 MI355X (MNIST-shape fp32 b128); % HBM / MFMA peak",
@@ -427,15 +382,18 @@ def main():
                                "training steps (1568 -> 30x100, mask density 0.1, rewiring every 15th step)",
                    "batch": BATCH, "in_features": n, "hypercolumns": H, "minicolumns": MC,
                    "samples": args.samples},
+        "windows": windows,
         "roofline": {"bound": "hbm", "kernel": "k_train_fused", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(),
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "traffic_note": traffic_note,
                      "algorithmic_bytes_per_launch": alg_bytes,
                      "bytes_the_kernel_must_move_at_this_mask_density": min_bytes,
-                     "avg_launch_us": tw["avg_us"]},
+                     "avg_launch_us": tw["avg_us"],
+                     "trace_gemm_tflops": gemm_tflops, "trace_gemm_frac_of_mfma_peak": gemm_tflops / 157.3},
         "mfma": {"kernel": "k_forward_rows", "flops_per_launch_connected_rows_only": fwd_flops,
                  "achieved_tflops": fwd_tflops, "peak_tflops": 157.3,
                  "frac": fwd_tflops / 157.3, "avg_launch_us": fwd["avg_us"],
-                 "trace_gemm_tflops_in_fused_kernel": 2.0 * BATCH * n * m / (tw["avg_us"] * 1e-6) / 1e12},
+                 "trace_gemm_tflops_in_fused_kernel": gemm_tflops},
         "kernels": prof,
         "event_bracket_overhead_us": {"calibrated": bracket_us,
                                       "empty_bracket": run.lib.sb_profile_bracket_overhead_us()},
@@ -446,10 +404,359 @@ def main():
         },
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(x, y, budget_s=args.cpu_baseline_seconds)
+        st = initial_state()
+        result["cpu_baseline"] = cpu_baseline(x, st, H, MC, BATCH, HP["l1_taupdt"], np.float32,
+                                              budget_s=args.cpu_baseline_seconds)
     else:
         result["cpu_baseline"] = None
-    print(json.dumps(result))
+    if not args.no_other_configs:
+        result["other_configs"] = {}
+        for name in [w for w in args.other_configs.split(",") if w]:
+            steps, warm = SHORT_RUNS[name]
+            r = large_workload(name, steps, warm, with_cpu=not args.no_cpu_baseline)
+            result["other_configs"][name] = {k: r[k] for k in ("config", "value", "unit", "ms_per_step", "steps",
+                                                               "warmup", "windows", "dtype", "roofline", "mfma",
+                                                               "cpu_baseline")}
+    return result
+
+
+# Other layer shapes, run through the same network path (one structural-plasticity layer, data resident in
+# HBM, first epoch: no rewiring).  in_features, hypercolumns, minicolumns, batch, mask density, dtype,
+# samples kept on the device (an epoch of the run cycles through them), fraction of non-zero inputs,
+# seconds of CPU baseline (None: not run).
+LARGE = {
+    "dense": dict(n=1568, h=30, mc=100, batch=128, density=1.0, dtype=np.float32, samples=60000, nonzero=0.19,
+                  cpu_s=3.0,
+                  what="configs[0]: single hidden layer 1568 -> 30x100, float32, batch 128, dense (no mask), one epoch"),
+    "stl10": dict(n=55296, h=200, mc=100, batch=256, density=0.05, dtype=np.float32, samples=5000, nonzero=1.0,
+                  cpu_s=0.0,
+                  what="configs[3]: STL-10-shaped layer 55296 -> 200x100, float32, batch 256, mask density 0.05"),
+    "largest": dict(n=65536, h=1000, mc=100, batch=1024, density=1.0, dtype=np.float32, samples=4096, nonzero=0.2,
+                    cpu_s=None,
+                    what="configs[4]: 65536 -> 1000x100, float32, batch 1024, binary inputs, dense mask"),
+    "mnist15x200": dict(n=1568, h=15, mc=200, batch=128, density=0.1, dtype=np.float32, samples=60000, nonzero=0.19,
+                        cpu_s=3.0,
+                        what="the reference example script's own MNIST layer: 1568 -> 15x200, float32, batch 128, "
+                             "mask density 0.1"),
+    "wide64": dict(n=1568, h=100, mc=100, batch=512, density=0.1, dtype=np.float64, samples=60000, nonzero=0.19,
+                   cpu_s=3.0,
+                   what="configs[2]: 1568 -> 100x100, float64, batch 512, mask density 0.1"),
+}
+# (timed steps per window, warm-up steps) of the short runs inside the default invocation
+SHORT_RUNS = {"dense": (100, 40), "wide64": (40, 20), "stl10": (10, 4), "largest": (3, 2)}
+
+
+def large_inputs(name):
+    cfg = LARGE[name]
+    n, ns, dt = cfg["n"], cfg["samples"], cfg["dtype"]
+    rng = np.random.default_rng(1000 + len(name))
+    if name == "largest":
+        x = (rng.random((ns, n), dtype=np.float32) < cfg["nonzero"]).astype(dt)
+    else:
+        half = n // 2
+        px = rng.random((ns, half), dtype=np.float32)
+        if cfg["nonzero"] < 1.0:
+            px *= rng.random((ns, half), dtype=np.float32) < cfg["nonzero"]
+        x = np.concatenate([px, 1.0 - px], axis=1).astype(dt)
+    wmask = None
+    if cfg["density"] < 1.0:
+        wmask = (rng.random((n, cfg["h"]), dtype=np.float32) < cfg["density"]).astype(np.uint8)
+    return x, wmask, rng
+
+
+def large_cpu_baseline(name, x, wmask):
+    """CPU baseline of one of the other configurations: same shapes and data, state as the GPU run starts
+    from (weights: one block of normal draws repeated, which costs the CPU the same work)."""
+    cfg = LARGE[name]
+    if cfg["cpu_s"] is None:
+        return {"value": None, "unit": "samples/s", "kind": "port",
+                "reason": "not run: Cij and W alone need 52 GB of host memory and a step takes minutes "
+                          "(about 27 TFLOP of scalar-vector loops per step)"}
+    n, h, mc, dt = cfg["n"], cfg["h"], cfg["mc"], cfg["dtype"]
+    m = h * mc
+    rng = np.random.default_rng(5)
+    block = (0.1 * rng.standard_normal(1 << 20)).astype(dt)
+    st = {"weights": np.resize(block, (n, m)), "bias": (0.1 * rng.random(m)).astype(dt),
+          "Ci": np.ones(n, dtype=dt), "Cj": np.full(m, 1.0 / mc, dtype=dt), "Cij": np.full((n, m), 1.0 / mc, dtype=dt),
+          "kbi": np.ones(m, dtype=dt),
+          "wmask": wmask if wmask is not None else np.ones((n, h), dtype=np.uint8)}
+    st["weights"] = np.ascontiguousarray(st["weights"] * np.repeat(st["wmask"], mc, axis=1).astype(dt)
+                                         if wmask is not None and n * m < (1 << 28) else st["weights"])
+    tau = HP["l1_taupdt"] * np.sqrt(cfg["batch"] / 128.0)
+    big = n * m > (1 << 28)
+    return cpu_baseline(x, st, h, mc, cfg["batch"], tau, dt, budget_s=cfg["cpu_s"], min_steps=1,
+                        rewire_period=0, warm=not big)
+
+
+def large_workload(name, steps, warmup, with_cpu=True):
+    """Training steps of one structural-plasticity layer of a LARGE shape; returns the result line."""
+    from streambrain_amd import _capi
+    cfg = LARGE[name]
+    n, h, mc, batch, dt = cfg["n"], cfg["h"], cfg["mc"], cfg["batch"], cfg["dtype"]
+    m, ns, es = h * mc, cfg["samples"], np.dtype(cfg["dtype"]).itemsize
+    x, wmask, rng = large_inputs(name)
+    lib = _capi.lib()
+    _capi.init(0)
+    c = _capi.check
+    net = ctypes.c_void_p()
+    c(lib.sb_net_create(ctypes.byref(net), 0 if dt == np.float32 else 1))
+    tau = HP["l1_taupdt"] * np.sqrt(batch / 128.0)
+    c(lib.sb_net_add_plastic_layer(net, n, h, mc, tau, HP["l1_pmin"], HP["l1_khalf"], HP["l1_taubdt"], 1.0,
+                                   1.0 / mc, 1.0 / mc))
+    # a (never trained) output layer behind it, so that the layer trains on its own activation
+    c(lib.sb_net_add_dense_layer(net, m, 1, N_OUT, HP["l2_taupdt"], 1.0 / mc, 1.0 / N_OUT, 1.0 / mc / N_OUT))
+    connected = n * h
+    if wmask is not None:
+        connected = int(np.count_nonzero(wmask))
+        c(lib.sb_net_set_layer_state(net, 0, b"wmask", wmask.ctypes.data, wmask.nbytes))
+    c(lib.sb_net_set_training_data(net, x.ctypes.data, None, ns, n, 0))
+    nb = (ns + batch - 1) // batch
+
+    def run(first, count):
+        done = 0
+        for epoch, fb, take in batch_plan(first, count, nb):
+            perm = rng.permutation(ns).astype(np.int64) if fb == 0 else None
+            hc = rng.permutation(h).astype(np.int64)
+            c(lib.sb_net_train_batches(net, 0, batch, perm.ctypes.data if perm is not None else None,
+                                       hc.ctypes.data, 0, fb, take, 0))
+            done += sum(min(batch, ns - b * batch) for b in range(fb, fb + take))
+        return done
+
+    warmup = max(warmup, 1)
+    run(0, warmup)
+    c(lib.sb_sync())
+    times, samples_of, first = [], [], warmup
+    for _ in range(3):
+        t0 = time.perf_counter()
+        samples_of.append(run(first, steps))
+        c(lib.sb_sync())
+        times.append(time.perf_counter() - t0)
+        first += steps
+    mid, windows = window_stats(times, samples_of, steps)
+    dt_s, samples = times[mid], samples_of[mid]
+    c(lib.sb_profile_start())
+    n_prof = min(steps, nb)
+    run(first, n_prof)
+    c(lib.sb_profile_stop())
+    kernels, raw_ms, brackets = read_profile(lib, c)
+    bracket_us = calibrate_brackets(kernels, raw_ms, brackets, dt_s * n_prof / steps)
+    c(lib.sb_net_destroy(net))
+    tw = kernels.get("train_fused", {"avg_us": float("nan")})["avg_us"] * 1e-6
+    fw = kernels.get("forward", {"avg_us": float("nan")})["avg_us"] * 1e-6
+    dname = "f32" if dt == np.float32 else "f64"
+    peak = MFMA_PEAK_TFLOPS[dname]
+    gemm = 2.0 * batch * n * m  # the Cij trace GEMM of a full batch
+    fwd_flops = 2.0 * batch * connected * mc if cfg["density"] <= 0.5 else gemm
+    stream_bytes = 3 * es * n * m
+    # which roof bounds the fused kernel: its GEMM at the MFMA peak against its 3 s N M stream at the HBM peak
+    mfma_bound = gemm / (peak * 1e12) >= stream_bytes / (HBM_PEAK_GBS * 1e9)
+    if mfma_bound:
+        roofline = {"bound": "mfma", "kernel": "k_train_fused", "achieved": gemm / tw / 1e12, "peak": peak,
+                    "unit": "TFLOP/s", "frac": gemm / tw / 1e12 / peak, "traffic": None,
+                    "algorithmic_flops_per_launch": gemm, "avg_launch_us": tw * 1e6,
+                    "bytes_3sNM_per_launch": stream_bytes, "achieved_GBps_on_3sNM": stream_bytes / tw / 1e9}
+    else:
+        roofline = {"bound": "hbm", "kernel": "k_train_fused", "achieved": stream_bytes / tw / 1e9,
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": stream_bytes / tw / 1e9 / HBM_PEAK_GBS,
+                    "traffic": None, "algorithmic_bytes_per_launch": stream_bytes, "avg_launch_us": tw * 1e6,
+                    "trace_gemm_tflops": gemm / tw / 1e12, "trace_gemm_frac_of_mfma_peak": gemm / tw / 1e12 / peak}
+    return {
+        "metric": "train samples/sec on 1 MI355X; % HBM / MFMA peak",
+        "value": samples / dt_s, "unit": "samples/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": 1e3 * dt_s / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dname, "data": "synthetic",
+        "config": {"workload": cfg["what"], "batch": batch, "in_features": n, "hypercolumns": h,
+                   "minicolumns": mc, "samples": ns},
+        "windows": windows,
+        "roofline": roofline,
+        "mfma": {"kernel": "k_forward_rows" if cfg["density"] <= 0.5 else "k_forward",
+                 "flops_per_launch": fwd_flops, "achieved_tflops": fwd_flops / fw / 1e12, "peak_tflops": peak,
+                 "frac": fwd_flops / fw / 1e12 / peak, "avg_launch_us": fw * 1e6},
+        "kernels": kernels, "event_bracket_overhead_us": {"calibrated": bracket_us},
+        "cpu_baseline": large_cpu_baseline(name, x, wmask) if with_cpu else None}
+
+
+# ------------------------------------------------------------------------- counters, peaks, summaries
+def kernel_source_stamp():
+    """sha256 over the sources of the dominant kernel: a counter summary in profiles/ names the stamp of
+    the sources it was measured with."""
+    hsh = hashlib.sha256()
+    for f in KERNEL_SOURCES:
+        hsh.update(open(os.path.join(ROOT, "streambrain_amd", "csrc", f), "rb").read())
+    return hsh.hexdigest()[:16]
+
+
+def measured_traffic():
+    """HBM bytes per launch of the dominant kernel, as measured with rocprofv3 --pmc FETCH_SIZE /
+    WRITE_SIZE and recorded in profiles/ (lines `traffic_bytes_per_launch: N`, `kernel_source_stamp: S`);
+    (None, why) when there is no summary or it was measured with other kernel sources."""
+    traffic = stamp = None
+    try:
+        for line in open(PMC_PROFILE):
+            if line.startswith("traffic_bytes_per_launch:"):
+                traffic = float(line.split(":", 1)[1])
+            if line.startswith("kernel_source_stamp:"):
+                stamp = line.split(":", 1)[1].strip()
+    except OSError:
+        return None, "no counter summary in profiles/"
+    if traffic is None:
+        return None, "no traffic line in the counter summary"
+    if stamp != kernel_source_stamp():
+        return None, "the counter summary in profiles/ was measured with other kernel sources"
+    return traffic, "rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain copy (profiles/)"
+
+
+def copy_calibration(nbytes=64 << 20, copies=6):
+    from streambrain_amd import _capi
+    from streambrain_amd._capi import DeviceArray
+    _capi.init(0)
+    lib = _capi.lib()
+    src, dst = DeviceArray((nbytes,), np.uint8), DeviceArray((nbytes,), np.uint8)
+    _capi.check(lib.sb_fill_bytes(src.ptr, 1, nbytes))
+    _capi.check(lib.sb_fill_bytes(dst.ptr, 2, nbytes))
+    for _ in range(copies):
+        _capi.check(lib.sb_memcpy_d2d(dst.ptr, src.ptr, nbytes))
+    _capi.check(lib.sb_sync())
+    print(json.dumps({"copy_calibration": {"copies": copies, "bytes_read_per_copy": nbytes,
+                                           "bytes_written_per_copy": nbytes}}))
+    return 0
+
+
+def achievable_peaks():
+    """What the box reaches in practice, next to the published peaks: device-to-device copies of three
+    sizes (bytes read + written per second) and MFMA-only kernels in float and double."""
+    from streambrain_amd import _capi
+    from streambrain_amd._capi import DeviceArray
+    _capi.init(0)
+    lib, c = _capi.lib(), _capi.check
+    out = {"hbm_peak_GBps_published": HBM_PEAK_GBS, "copies": [], "mfma": []}
+    for nbytes in (32 << 20, 128 << 20, 2 << 30):
+        src, dst = DeviceArray((nbytes,), np.uint8), DeviceArray((nbytes,), np.uint8)
+        c(lib.sb_fill_bytes(src.ptr, 1, nbytes))
+        c(lib.sb_fill_bytes(dst.ptr, 2, nbytes))
+        reps = max(4, min(200, (8 << 30) // nbytes))
+        best = float("inf")
+        for _ in range(3):
+            c(lib.sb_sync())
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                c(lib.sb_memcpy_d2d(dst.ptr, src.ptr, nbytes))
+            c(lib.sb_sync())
+            best = min(best, (time.perf_counter() - t0) / reps)
+        out["copies"].append({"bytes": nbytes, "copies_timed": reps, "us_per_copy": 1e6 * best,
+                              "GBps_read_plus_written": 2 * nbytes / best / 1e9,
+                              "frac_of_published_peak": 2 * nbytes / best / 1e9 / HBM_PEAK_GBS})
+        src.free()
+        dst.free()
+    for dtype, name in ((0, "f32"), (1, "f64")):
+        flops = ctypes.c_double(0)
+        c(lib.sb_probe_mfma(dtype, 2048, 1000, ctypes.byref(flops)))  # warm-up
+        c(lib.sb_sync())
+        for iters, what in ((1000, "short launch (a few ms)"), (20000, "long launch (tens of ms)")):
+            best = float("inf")
+            for _ in range(3):
+                t0 = time.perf_counter()
+                c(lib.sb_probe_mfma(dtype, 2048, iters, ctypes.byref(flops)))
+                c(lib.sb_sync())
+                best = min(best, time.perf_counter() - t0)
+            out["mfma"].append({"dtype": name, "instruction": "16x16x4", "workgroups": 2048, "what": what,
+                                "flops": flops.value, "ms": 1e3 * best, "TFLOPps": flops.value / best / 1e12,
+                                "published_peak_TFLOPps": MFMA_PEAK_TFLOPS[name],
+                                "frac_of_published_peak": flops.value / best / 1e12 / MFMA_PEAK_TFLOPS[name]})
+    print(json.dumps({"achievable_peaks": out}))
+    return 0
+
+
+def _pmc_medians(directory):
+    import collections
+    import csv
+    import glob
+    import re
+    files = []
+    for d in directory.split(","):  # several runs' directories, comma-separated
+        files += sorted(glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True))
+    res = collections.defaultdict(lambda: collections.defaultdict(list))
+    for f in files:
+        for row in csv.DictReader(open(f)):
+            k = re.sub(r"^void sb::", "", re.sub(r"\(.*", "", row["Kernel_Name"]))
+            res[k][row["Counter_Name"]].append(float(row["Counter_Value"]))
+    return {k: {c: (len(v), sorted(v)[len(v) // 2]) for c, v in d.items()} for k, d in res.items()}
+
+
+def pmc_summary(directory, calibration=None):
+    """Per-kernel medians of the counters in the rocprofv3 --pmc output below `directory` (csv format) as
+    text.  With `calibration` (the output of the same counters over `bench.py --copy-calibration`),
+    FETCH_SIZE / WRITE_SIZE (KiB per dispatch) are scaled by what they read for the plain 64 MiB copies and
+    the traffic of the fused training kernel is printed as the line bench.py reads back."""
+    med = _pmc_medians(directory)
+    print(f"kernel_source_stamp: {kernel_source_stamp()}")
+    scale = {}
+    if calibration:
+        cal = _pmc_medians(calibration)
+        copy = next((d for k, d in cal.items() if "copyBuffer" in k or "copy" in k.lower()), None)
+        if copy:
+            for cname in ("FETCH_SIZE", "WRITE_SIZE"):
+                if cname in copy and copy[cname][1] > 0:
+                    scale[cname] = 65536.0 / copy[cname][1]
+                    print(f"calibration: plain device copy of 64 MiB reads {cname} = {copy[cname][1]:.1f} KiB "
+                          f"-> scale {scale[cname]:.4f}")
+    for k, d in sorted(med.items()):
+        print(k)
+        for cname, (n, v) in sorted(d.items()):
+            extra = f"  = {v * 1024 * scale[cname] / 1e6:10.2f} MB per launch" if cname in scale else ""
+            print(f"   {cname:32s} launches={n:5d} median={v:16.1f}{extra}")
+    fused = [d for k, d in med.items() if k.startswith("k_train_fused")]
+    if fused and len(scale) == 2 and all(c in fused[0] for c in scale):
+        total = sum(fused[0][c][1] * 1024 * scale[c] for c in scale)
+        print(f"traffic_bytes_per_launch: {total:.0f}")
+    return 0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=938)
+    ap.add_argument("--warmup", type=int, default=60)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="leave out the short runs of the other four configurations")
+    ap.add_argument("--other-configs", default="dense,wide64,stl10,largest",
+                    help="which of the other configurations the default run adds (comma-separated)")
+    ap.add_argument("--cpu-baseline-seconds", type=float, default=15.0,
+                    help="length of the headline CPU baseline's sample")
+    ap.add_argument("--samples", type=int, default=N_SAMPLES)
+    ap.add_argument("--workload", choices=["mnist"] + sorted(LARGE), default="mnist",
+                    help="mnist (default): the headline configuration with short runs of the others; the "
+                         "others: one layer of that shape alone (--steps defaults to two epochs of its "
+                         "resident samples)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run six 64 MiB device-to-device copies: the known-size kernel that "
+                         "hardware counter readings (FETCH_SIZE, WRITE_SIZE) are scaled by")
+    ap.add_argument("--achievable-peaks", action="store_true",
+                    help="only measure device-copy bandwidth and MFMA-only kernels (what the box reaches "
+                         "next to the published peaks)")
+    ap.add_argument("--pmc-summary", metavar="DIR", help="summarise rocprofv3 --pmc csv output below DIR")
+    ap.add_argument("--pmc-calibration", metavar="DIR",
+                    help="with --pmc-summary: the same counters over `bench.py --copy-calibration`")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
+              "(the path is not sharded across devices)", file=sys.stderr)
+        return 2
+    if args.pmc_summary:
+        return pmc_summary(args.pmc_summary, args.pmc_calibration)
+    if args.copy_calibration:
+        return copy_calibration()
+    if args.achievable_peaks:
+        return achievable_peaks()
+    if args.workload != "mnist":
+        cfg = LARGE[args.workload]
+        nb = (cfg["samples"] + cfg["batch"] - 1) // cfg["batch"]
+        steps = args.steps if "--steps" in sys.argv else (nb if nb > 100 else 2 * nb)
+        print(json.dumps(large_workload(args.workload, steps, args.warmup if "--warmup" in sys.argv else nb,
+                                        with_cpu=not args.no_cpu_baseline)))
+        return 0
+    print(json.dumps(headline(args)))
     return 0
 
 

@@ -59,6 +59,7 @@ _PLAIN_SIGS = {
     "sb_net_training_done": [_P],
     "sb_net_train_epoch": [_P, _I, _L, _P, _P, _L],
     "sb_net_train_batches": [_P, _I, _L, _P, _P, _L, _L, _L, _I],
+    "sb_probe_mfma": [_I, _L, _L, ctypes.POINTER(_D)],
     "sb_profile_start": [],
     "sb_profile_stop": [],
     "sb_profile_kernels": [],

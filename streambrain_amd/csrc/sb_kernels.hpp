@@ -414,6 +414,25 @@ __global__ __launch_bounds__(256) void k_gather_rows_blocked(T *dst, T *plain, c
   }
 }
 
+// Matrix-core probe: every wavefront issues `iters` rounds of eight independent 16x16x4 MFMAs (nothing else
+// in the loop), so launches / time gives the rate the matrix cores reach on this element type in practice.
+template <typename T>
+__global__ __launch_bounds__(256) void k_mfma_probe(T *sink, long iters) {
+  using R = Real<T>;
+  typename R::acc_t acc[8];
+#pragma unroll
+  for (int k = 0; k < 8; k++) acc[k] = typename R::acc_t{T(k), 0, 0, 0};
+  const T a = T(1) + T(threadIdx.x) * T(1e-6), b = T(1) - T(threadIdx.x) * T(1e-6);
+  for (long i = 0; i < iters; i++) {
+#pragma unroll
+    for (int k = 0; k < 8; k++) acc[k] = R::mfma(a, b, acc[k]);
+  }
+  T s = T(0);
+#pragma unroll
+  for (int k = 0; k < 8; k++) s += acc[k][0] + acc[k][1] + acc[k][2] + acc[k][3];
+  if (s == T(-1)) sink[0] = s;  // never true: keeps the loop
+}
+
 template <int UNUSED = 0>
 __global__ __launch_bounds__(256) void k_fill_bytes(uint8_t *dst, uint8_t value, size_t bytes) {
   const size_t stride = (size_t)gridDim.x * 256;

@@ -127,6 +127,9 @@ int launch_gather_rows(hipStream_t st, T *dst, const T *src, const int64_t *idx,
 template <typename T>
 int launch_gather_rows_blocked(hipStream_t st, T *dst, T *plain, const T *src, const int64_t *idx, long rows,
                                long cols);
+// `workgroups` workgroups of four wavefronts, each wavefront 8 * iters MFMAs of 2 * 16 * 16 * 4 flops.
+template <typename T>
+int launch_mfma_probe(hipStream_t st, T *sink, long workgroups, long iters);
 template <typename T>
 int launch_fill(hipStream_t st, T *dst, T value, size_t n);
 int launch_fill_bytes(hipStream_t st, void *dst, int value, size_t bytes);

@@ -478,6 +478,15 @@ int launch_gather_rows_blocked(hipStream_t st, T *dst, T *plain, const T *src, c
 }
 
 template <typename T>
+int launch_mfma_probe(hipStream_t st, T *sink, long workgroups, long iters) {
+  SB_REQUIRE(sink, "null pointer");
+  SB_REQUIRE(workgroups > 0 && workgroups < (1L << 31) && iters > 0 && iters <= (1L << 24), "bad sizes");
+  hipLaunchKernelGGL((k_mfma_probe<T>), dim3((unsigned)workgroups), dim3(256), 0, st, sink, iters);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
 int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
   if (n == 0) return 0;
   SB_REQUIRE(dst, "null pointer");
@@ -518,6 +527,7 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
   template int launch_argmax_rows<T>(hipStream_t, const T *, const T *, long, long, int32_t *,        \
                                      unsigned long long *);                                           \
   template int launch_gather_rows<T>(hipStream_t, T *, const T *, const int64_t *, long, long);       \
+  template int launch_mfma_probe<T>(hipStream_t, T *, long, long);                                    \
   template int launch_fill<T>(hipStream_t, T *, T, size_t);
 
 }  // namespace sb

@@ -994,6 +994,21 @@ int sb_net_train_epoch(sb_net *net, int layer, long maximal_batch_size, const in
                               nb, 1);
 }
 
+// Matrix-core probe (see k_mfma_probe); *flops receives the floating-point operations of the launch.
+static int mfma_probe(int dtype, long workgroups, long iters, double *flops) {
+  SB_READY();
+  SB_REQUIRE(dtype == SB_F32 || dtype == SB_F64, "dtype must be SB_F32 or SB_F64");
+  int rc = ensure_trace_scratch(1);
+  if (rc) return rc;
+  rc = dtype == SB_F32 ? launch_mfma_probe<float>(g_ctx.stream, (float *)g_ctx.trace_next, workgroups, iters)
+                       : launch_mfma_probe<double>(g_ctx.stream, (double *)g_ctx.trace_next, workgroups, iters);
+  if (!rc && flops) *flops = (double)workgroups * 4.0 * (double)iters * 8.0 * 2.0 * 16 * 16 * 4;
+  return rc;
+}
+int sb_probe_mfma(int dtype, long workgroups, long iters, double *flops) {
+  return mfma_probe(dtype, workgroups, iters, flops);
+}
+
 int sb_profile_start(void) {
   SB_READY();
   SB_HIP(hipStreamSynchronize(g_ctx.stream));

@@ -22,7 +22,8 @@ def _run(*args):
 
 
 def test_headline_line_short_run():
-    b = _run("--steps", "60", "--warmup", "10", "--samples", "8960", "--cpu-baseline-seconds", "2")
+    b = _run("--steps", "60", "--warmup", "10", "--samples", "8960", "--cpu-baseline-seconds", "2",
+             "--other-configs", "dense")
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
                 "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
         assert key in b, key
@@ -35,13 +36,25 @@ def test_headline_line_short_run():
     assert r["bound"] == "hbm" and r["unit"] == "GB/s" and r["peak"] == 8000.0
     assert r["frac"] == pytest.approx(r["achieved"] / r["peak"], rel=1e-9) and 0.0 < r["frac"] < 1.0
     assert r["achieved"] == pytest.approx(r["algorithmic_bytes_per_launch"] / (r["avg_launch_us"] * 1e-6) / 1e9, rel=1e-6)
+    # the counter summary in profiles/ belongs to the kernel sources of this tree
+    assert r["traffic"] is not None, r["traffic_note"]
+    assert 0.5 * r["algorithmic_bytes_per_launch"] < r["traffic"] < 2 * r["algorithmic_bytes_per_launch"]
+    w = b["windows"]
+    assert w["count"] >= 3 and w["ms_per_step_min"] <= w["ms_per_step_median"] <= w["ms_per_step_max"]
+    assert b["ms_per_step"] == pytest.approx(w["ms_per_step_median"], rel=1e-9)
     c = b["cpu_baseline"]
     assert c["kind"] == "port" and c["cores"] >= 1 and c["value"] > 0 and c["unit"] == "samples/s"
     assert b["value"] > c["value"]
+    assert set(c["ms_per_step_by_function"]) == {"forward_blas", "softmax_numpy", "traces_and_weights", "bias", "mask"}
+    assert sum(c["ms_per_step_by_function"].values()) <= c["ms_per_step"] * 1.001
+    assert c["host"]["cpu_model"] and c["host"]["threads_used"] >= 1
+    o = b["other_configs"]["dense"]
+    assert "configs[0]" in o["config"]["workload"] and o["value"] > 0 and 0.0 < o["roofline"]["frac"] < 1.0
+    assert o["cpu_baseline"]["value"] > 0
 
 
 def test_other_workload_line():
-    b = _run("--workload", "dense", "--steps", "40", "--warmup", "10")
+    b = _run("--workload", "dense", "--steps", "40", "--warmup", "10", "--no-cpu-baseline")
     assert b["n_gpus"] == 1 and b["dtype"] == "f32" and b["cpu_baseline"] is None
     assert b["roofline"]["bound"] in ("hbm", "mfma") and 0.0 < b["roofline"]["frac"] < 1.0
     assert "configs[0]" in b["config"]["workload"]
