@@ -229,7 +229,7 @@ int sb_net_training_done(sb_net *net);
  * When n_batches / (H + 1) is zero the reference divides by zero; here no rewiring happens.
  * While the last layer trains, the layers below it do not change: their activations of the training set
  * are computed in its first epoch and kept (two copies of [n_samples, its input width], as long as
- * they stay below 16 GiB) until a lower layer trains, state is written or the training set is replaced.
+ * they stay below 16 GiB and half of the free device memory) until a lower layer trains, state is written or the training set is replaced.
  * Asynchronous: returns once the epoch is enqueued. */
 int sb_net_train_epoch(sb_net *net, int layer, long maximal_batch_size,
                        const int64_t *h_sample_perm, const int64_t *h_hc_perm, long epoch_index);
@@ -258,6 +258,19 @@ int sb_net_predict(sb_net *net, const void *h_images, long n_samples, long n_fea
  * last_layer [n_rows, M_last] is copied to h_act.  Synchronous. */
 int sb_net_forward(sb_net *net, const void *h_images, long n_rows, long n_features, int last_layer,
                    long maximal_batch_size, void *h_act);
+
+/* The layer-level calls of the DSL on one layer of the network, on host arrays in the network dtype
+ * (_cpu_base_backend.py:44-51,126-133 compute_activation; cpu_backend.py:13-18,29-52 train_step and
+ * train_finalize).  Synchronous.
+ *   sb_net_layer_activation      h_act[n_rows, M] = softmax_hc(h_inputs[n_rows, N] . W + bias) of `layer`
+ *   sb_net_layer_train_step      one training step of `layer` on inputs [n_rows, N] and outputs [n_rows, M]
+ *                                (its own activation, or the labels for the last layer); hypercolumn >= 0
+ *                                also rewires that hypercolumn (structural-plasticity layers), -1: none
+ *   sb_net_layer_train_finalize  dense layers: bias from Cj; structural-plasticity layers: nothing */
+int sb_net_layer_activation(sb_net *net, int layer, const void *h_inputs, long n_rows, void *h_act);
+int sb_net_layer_train_step(sb_net *net, int layer, const void *h_inputs, const void *h_outputs, long n_rows,
+                            long hypercolumn);
+int sb_net_layer_train_finalize(sb_net *net, int layer);
 
 /* ---- per-kernel timing -------------------------------------------------------------------------
  * Between sb_profile_start and sb_profile_stop every kernel launch of the library is bracketed by HIP

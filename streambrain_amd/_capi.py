@@ -59,6 +59,9 @@ _PLAIN_SIGS = {
     "sb_net_training_done": [_P],
     "sb_net_train_epoch": [_P, _I, _L, _P, _P, _L],
     "sb_net_train_batches": [_P, _I, _L, _P, _P, _L, _L, _L, _I],
+    "sb_net_layer_activation": [_P, _I, _P, _L, _P],
+    "sb_net_layer_train_step": [_P, _I, _P, _P, _L, _L],
+    "sb_net_layer_train_finalize": [_P, _I],
     "sb_probe_mfma": [_I, _L, _L, ctypes.POINTER(_D)],
     "sb_profile_start": [],
     "sb_profile_stop": [],

@@ -36,6 +36,7 @@ except ImportError as exc:  # no fallback: the GPU module is the backend
 
 _backend.initialize(int(os.environ.get("BCPNN_HIP_DEVICE", "0")))
 
+
 _FLOAT_STATE = ("weights", "bias", "Ci", "Cj", "Cij")
 
 
@@ -92,6 +93,29 @@ class _DeviceLayer:
         if self._net is None:
             for name in type(self)._state_names:
                 self._host[name] = self._host[name].astype(dtype)
+
+    # ---- the layer-level calls of the reference's layers (_cpu_base_backend.py:44-68, 126-172;
+    # cpu_backend.py:13-18, 29-52), on the layer's state in HBM
+    def _attached(self, what):
+        if self._net is None:
+            raise RuntimeError(f"{what}: the layer's state lives on the GPU once it has been added to a "
+                               "Network (Network.add_layer); add it first")
+        return self._net
+
+    def compute_activation(self, inputs):
+        net = self._attached("compute_activation")
+        return net.layer_activation(self._index, np.ascontiguousarray(inputs, dtype=self.dtype))
+
+    def train_step(self, inputs, outputs, hypercolumn=None):
+        net = self._attached("train_step")
+        if hypercolumn is not None and not isinstance(self, StructuralPlasticityLayer):
+            raise TypeError("train_step: only a StructuralPlasticityLayer takes a hypercolumn")
+        net.layer_train_step(self._index, np.ascontiguousarray(inputs, dtype=self.dtype),
+                             np.ascontiguousarray(outputs, dtype=self.dtype),
+                             -1 if hypercolumn is None else int(hypercolumn))
+
+    def train_finalize(self):
+        self._attached("train_finalize").layer_train_finalize(self._index)
 
     def _upload(self, net, index):
         for name, value in self._host.items():

@@ -192,6 +192,27 @@ class PyNetwork {
     return out;
   }
 
+  // layer-level calls of the DSL (compute_activation, train_step, train_finalize of one layer)
+  py::array_t<REAL> layer_activation(int layer, carray<REAL> inputs) {
+    const Shape &s = shape_of(layer);
+    if (inputs.ndim() != 2 || inputs.shape(1) != s.n_inputs)
+      throw std::runtime_error("compute_activation: inputs [rows, in_features] expected");
+    py::array_t<REAL> out({(py::ssize_t)inputs.shape(0), (py::ssize_t)(s.hypercolumns * s.minicolumns)});
+    if (inputs.shape(0) > 0)
+      check(sb_net_layer_activation(net_, layer, inputs.data(), inputs.shape(0), out.mutable_data()));
+    return out;
+  }
+
+  void layer_train_step(int layer, carray<REAL> inputs, carray<REAL> outputs, long hypercolumn) {
+    const Shape &s = shape_of(layer);
+    if (inputs.ndim() != 2 || outputs.ndim() != 2 || inputs.shape(0) != outputs.shape(0) ||
+        inputs.shape(1) != s.n_inputs || outputs.shape(1) != s.hypercolumns * s.minicolumns)
+      throw std::runtime_error("train_step: inputs [rows, in_features] and outputs [rows, out_features] expected");
+    check(sb_net_layer_train_step(net_, layer, inputs.data(), outputs.data(), inputs.shape(0), hypercolumn));
+  }
+
+  void layer_train_finalize(int layer) { check(sb_net_layer_train_finalize(net_, layer)); }
+
   void synchronize() { check(sb_sync()); }
   size_t n_layers() const { return shapes_.size(); }
 
@@ -219,6 +240,9 @@ void bind_network(py::module_ &m, const char *name) {
            py::arg("sample_perm"), py::arg("hc_perm"), py::arg("epoch"))
       .def("evaluate_counts", &N::evaluate_counts)
       .def("forward", &N::forward)
+      .def("layer_activation", &N::layer_activation)
+      .def("layer_train_step", &N::layer_train_step)
+      .def("layer_train_finalize", &N::layer_train_finalize)
       .def("predict", &N::predict)
       .def("seed", &N::seed)
       .def("synchronize", &N::synchronize)

@@ -18,11 +18,6 @@
 #pragma once
 #include "sb_common.hpp"
 
-// Hook for phase timing in development builds; expands to nothing in the library.
-#ifndef SB_PHASE_MARK
-#define SB_PHASE_MARK(n)
-#endif
-
 namespace sb {
 
 template <typename T>
@@ -130,8 +125,6 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
       }
   }
   __syncthreads();
-
-  SB_PHASE_MARK(2);
   // ---- bias (+ softmax): TPR threads per batch row, thread handles columns lr + TPR t
   constexpr int TPR = ForwardBias<T, NG, NWAVES>::TPR, PT = ForwardBias<T, NG, NWAVES>::PT;
   const int row = tid / TPR, lr = tid % TPR;
@@ -281,7 +274,6 @@ void k_forward(ForwardArgs<T> a) {
   T bv[ForwardBias<T, NG, NWAVES>::PT];
   ForwardBias<T, NG, NWAVES>::load(bv, a.bias, j0, ncol);
   const long nfull = a.N / KC;  // chunks with all KC reduction indices inside the matrix
-  SB_PHASE_MARK(0);
   {
     // Chunk `w` first; every later chunk of this wavefront is NWAVES chunks further on.  x and W are
     // reached through bounds-checked buffer windows that start at the chunk (a scalar base address,
@@ -354,14 +346,11 @@ void k_forward(ForwardArgs<T> a) {
       compute(xr[0], wr[0]);
     }
   }
-
-  SB_PHASE_MARK(1);
 #pragma unroll
   for (int r = 0; r < RB; r++) {
     if (r > 0) __syncthreads();  // the previous row block's sums have been read
     forward_finish<T, NG, FUSE, NWAVES, LW>(acc[r], bv, red, a.act, a.B, a.M, b0 + 16 * r, j0, ncol);
   }
-  SB_PHASE_MARK(3);
 }
 
 }  // namespace sb

@@ -83,7 +83,6 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
   const long j0 = ct * a.Mc;
   const long ncol = a.Mc;
   const int *list = ar.rows + ct * ar.cap;
-  SB_PHASE_MARK(0);
 
   // first segment of the list on its way before anything else
   constexpr int PT = SEG / (64 * NWAVES);  // entries per thread and segment
@@ -179,10 +178,6 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
     publish_segment(seg0);
     __syncthreads();
     request(w, xr[0], wr[0]);  // this wavefront's first chunk of the segment
-    SB_PHASE_MARK(12);
-#ifdef SB_PHASE_WAIT
-    SB_PHASE_WAIT();
-#endif
     // chunks w, w + NWAVES, ... of the segment that hold list entries: n of them (at least 1 in the
     // first segment, see above)
     const long left = (long)cnt - seg0;  // entries from the start of this segment
@@ -209,13 +204,11 @@ void k_forward_rows(ForwardRowsArgs<T> ar) {
     seg0 += SEG;
     __syncthreads();  // everyone is done with the staged segment
   }
-  SB_PHASE_MARK(1);
 #pragma unroll
   for (int r = 0; r < RB; r++) {
     if (r > 0) __syncthreads();  // the previous row block's sums have been read
     forward_finish<T, NG, true, NWAVES, LW>(acc[r], bv, red, a.act, a.B, a.M, b0 + 16 * r, j0, ncol);
   }
-  SB_PHASE_MARK(3);
 }
 
 }  // namespace sb

@@ -86,16 +86,16 @@ __global__ __launch_bounds__(256) void k_weights_from_traces(T *W, const T *Ci, 
   }
 }
 
-// omp.cc:322-335
+// omp.cc:322-335.  A row of W per workgroup and turn; the hypercolumn of a column is a multiplication by a
+// constant the host prepares (M < 2^31).
 template <typename T>
 __global__ __launch_bounds__(256) void k_apply_mask(T *W, const uint8_t *wmask, long N, long M, long H,
-                                                    long Mc) {
-  const long total = N * M;
-  const long stride = (long)gridDim.x * 256;
-  for (long e = (long)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
-    const long i = e / M;
-    const long j = e - i * M;
-    if (wmask[i * H + j / Mc] == 0) W[e] = T(0);
+                                                    FastDiv by_Mc) {
+  for (long i = blockIdx.x; i < N; i += gridDim.x) {
+    T *row = W + i * M;
+    const uint8_t *mrow = wmask + i * H;
+    for (unsigned j = threadIdx.x; j < (unsigned)M; j += 256)
+      if (mrow[by_Mc.div(j)] == 0) row[j] = T(0);
   }
 }
 

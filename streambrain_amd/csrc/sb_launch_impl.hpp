@@ -415,11 +415,11 @@ template <typename T>
 int launch_apply_mask(hipStream_t st, T *W, const uint8_t *wmask, long N, long H, long Mc) {
   SB_REQUIRE(W && wmask, "null pointer");
   SB_REQUIRE(N > 0 && H > 0 && Mc > 0, "sizes must be positive");
-  const long total = N * H * Mc;
-  const long blocks = cdiv(total, 256) < 8192 ? cdiv(total, 256) : 8192;
+  SB_REQUIRE(H * Mc < (1L << 31), "dimension too large");
+  const long blocks = N < 8192 ? N : 8192;
   ProfScope prof_(st, K_APPLY_MASK);
-  hipLaunchKernelGGL((k_apply_mask<T>), dim3((unsigned)blocks), dim3(256), 0, st, W, wmask, N, H * Mc,
-                     H, Mc);
+  hipLaunchKernelGGL((k_apply_mask<T>), dim3((unsigned)blocks), dim3(256), 0, st, W, wmask, N, H * Mc, H,
+                     FastDiv::of(Mc));
   SB_LAUNCH_CHECK();
   return 0;
 }

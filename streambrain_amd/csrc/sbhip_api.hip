@@ -360,8 +360,18 @@ static int layer_mask_replaced(Layer &L, const uint8_t *mask) {
   return launch_mask_rows(g_ctx.stream, L.rows, L.row_cnt, L.wmask, L.N, L.H, L.rows_cap, 0, L.H);
 }
 
-// Largest cache of frozen activations kept (bytes, both copies together); beyond it they are recomputed.
+// Largest cache of frozen activations kept (bytes, both copies together): at most 16 GiB, and at most half of
+// the device memory that is free when the cache is built; beyond it the activations are recomputed.
 static const size_t kFrozenCacheLimit = (size_t)16 << 30;
+static bool frozen_cache_affordable(size_t bytes) {
+  if (bytes > kFrozenCacheLimit) return false;
+  size_t free_b = 0, total_b = 0;
+  if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return bytes <= free_b / 2;
+}
 
 static int drop_frozen_cache(sb_net *net) {
   if (!net->Hc && !net->Hcp) {
@@ -381,8 +391,15 @@ static int build_frozen_cache(sb_net *net, int upto, long maxB) {
   const long Ns = net->Ns, Mo = net->layers[upto].M;
   int rc = drop_frozen_cache(net);
   if (rc) return rc;
-  SB_HIP(hipMalloc(&net->Hc, (size_t)Ns * Mo * sizeof(T)));
-  SB_HIP(hipMalloc(&net->Hcp, (size_t)Ns * Mo * sizeof(T)));
+  // without the memory for both copies the caller goes on uncached (Hc_layer stays -1): not an error
+  if (hipMalloc(&net->Hc, (size_t)Ns * Mo * sizeof(T)) != hipSuccess ||
+      hipMalloc(&net->Hcp, (size_t)Ns * Mo * sizeof(T)) != hipSuccess) {
+    (void)hipGetLastError();
+    net->Hcp = nullptr;
+    if (net->Hc) (void)hipFree(net->Hc);
+    net->Hc = nullptr;
+    return 0;
+  }
   for (long lo = 0; lo < Ns; lo += maxB) {
     const long B = lo + maxB <= Ns ? maxB : Ns - lo;
     const T *x = (const T *)net->X + lo * net->NF;
@@ -420,7 +437,8 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
   // a training step of a layer below the last changes what the cache was computed from
   if (!last && (rc = drop_frozen_cache(net))) return rc;
   const long Mprev = layer > 0 ? net->layers[layer - 1].M : 0;
-  const bool cache_fits = last && layer > 0 && 2 * (size_t)Ns * Mprev * sizeof(T) <= kFrozenCacheLimit;
+  const bool cache_fits = last && layer > 0 &&
+                          (net->Hc_layer == layer - 1 || frozen_cache_affordable(2 * (size_t)Ns * Mprev * sizeof(T)));
   if (permute) {
     SB_REQUIRE(h_sample_perm, "sample order missing");
     for (long r = 0; r < Ns; r++)
@@ -453,7 +471,9 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
         return rc;
     if (cache_fits) {
       if (net->Hc_layer != layer - 1 && (rc = build_frozen_cache<T>(net, layer - 1, maxB))) return rc;
-      if ((rc = launch_gather_rows<T>(st, (T *)net->Hcp, (const T *)net->Hc, net->d_perm, Ns, Mprev))) return rc;
+      if (net->Hc_layer == layer - 1 &&
+          (rc = launch_gather_rows<T>(st, (T *)net->Hcp, (const T *)net->Hc, net->d_perm, Ns, Mprev)))
+        return rc;
     } else if (last && (rc = drop_frozen_cache(net))) {
       return rc;
     }
@@ -576,6 +596,38 @@ static int net_forward_batches(sb_net *net, const void *h_images, const void *h_
     *correct = (int64_t)cnt;
   }
   if (rc) (void)hipStreamSynchronize(st);  // nothing in flight may still use the chunk buffers
+  return rc;
+}
+
+// compute_activation / train_step of ONE layer on host arrays (the layer-level calls of the DSL)
+template <typename T>
+static int net_layer_activation(sb_net *net, int layer, const void *h_in, long rows, void *h_act) {
+  Layer &L = net->layers[layer];
+  int rc = ensure_act(net, rows);
+  if (rc) return rc;
+  ScopedDeviceBuffer bX;
+  SB_HIP(hipMalloc(&bX.p, (size_t)rows * L.N * sizeof(T)));
+  SB_HIP(hipMemcpy(bX.p, h_in, (size_t)rows * L.N * sizeof(T), hipMemcpyHostToDevice));
+  rc = layer_forward<T>(net, L, (const T *)bX.p, rows);
+  if (!rc) SB_HIP(hipMemcpyAsync(h_act, L.act, (size_t)rows * L.M * sizeof(T), hipMemcpyDeviceToHost, g_ctx.stream));
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  return rc;
+}
+
+template <typename T>
+static int net_layer_train_step(sb_net *net, int layer, const void *h_in, const void *h_out, long rows, long h) {
+  Layer &L = net->layers[layer];
+  SB_REQUIRE(h < 0 || L.plastic, "only structural-plasticity layers rewire");
+  SB_REQUIRE(h < L.H, "hypercolumn index out of range");
+  int rc = drop_frozen_cache(net);  // the layer changes: what was computed from it is stale
+  if (rc) return rc;
+  ScopedDeviceBuffer bX, bY;
+  SB_HIP(hipMalloc(&bX.p, (size_t)rows * L.N * sizeof(T)));
+  SB_HIP(hipMalloc(&bY.p, (size_t)rows * L.M * sizeof(T)));
+  SB_HIP(hipMemcpy(bX.p, h_in, (size_t)rows * L.N * sizeof(T), hipMemcpyHostToDevice));
+  SB_HIP(hipMemcpy(bY.p, h_out, (size_t)rows * L.M * sizeof(T), hipMemcpyHostToDevice));
+  rc = layer_train_step<T>(L, (const T *)bX.p, (const T *)bY.p, rows, h);
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));  // the staging buffers go out of scope
   return rc;
 }
 
@@ -1007,6 +1059,39 @@ static int mfma_probe(int dtype, long workgroups, long iters, double *flops) {
 }
 int sb_probe_mfma(int dtype, long workgroups, long iters, double *flops) {
   return mfma_probe(dtype, workgroups, iters, flops);
+}
+
+int sb_net_layer_activation(sb_net *net, int layer, const void *h_inputs, long n_rows, void *h_act) {
+  SB_READY();
+  SB_REQUIRE(net && h_inputs && h_act, "null pointer");
+  SB_REQUIRE(layer >= 0 && layer < (int)net->layers.size(), "layer index out of range");
+  SB_REQUIRE(n_rows > 0, "sizes must be positive");
+  return net->dtype == SB_F32 ? net_layer_activation<float>(net, layer, h_inputs, n_rows, h_act)
+                              : net_layer_activation<double>(net, layer, h_inputs, n_rows, h_act);
+}
+
+int sb_net_layer_train_step(sb_net *net, int layer, const void *h_inputs, const void *h_outputs, long n_rows,
+                            long hypercolumn) {
+  SB_READY();
+  SB_REQUIRE(net && h_inputs && h_outputs, "null pointer");
+  SB_REQUIRE(layer >= 0 && layer < (int)net->layers.size(), "layer index out of range");
+  SB_REQUIRE(n_rows > 0, "sizes must be positive");
+  return net->dtype == SB_F32
+             ? net_layer_train_step<float>(net, layer, h_inputs, h_outputs, n_rows, hypercolumn)
+             : net_layer_train_step<double>(net, layer, h_inputs, h_outputs, n_rows, hypercolumn);
+}
+
+int sb_net_layer_train_finalize(sb_net *net, int layer) {
+  SB_READY();
+  SB_REQUIRE(net, "null pointer");
+  SB_REQUIRE(layer >= 0 && layer < (int)net->layers.size(), "layer index out of range");
+  Layer &L = net->layers[layer];
+  if (L.plastic) return 0;  // _cpu_base_backend.py:171-172
+  int rc = drop_frozen_cache(net);
+  if (rc) return rc;
+  return net->dtype == SB_F32
+             ? launch_update_bias<float>(g_ctx.stream, (float *)L.bias, (const float *)L.Cj, (float)(L.taupdt / 2), L.M)
+             : launch_update_bias<double>(g_ctx.stream, (double *)L.bias, (const double *)L.Cj, L.taupdt / 2, L.M);
 }
 
 int sb_profile_start(void) {

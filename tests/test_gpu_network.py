@@ -392,6 +392,52 @@ def test_rewiring_decisions_replayed_f32(hb):
         assert swapped > 0
 
 
+@pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-5), (np.float64, 1e-12)])
+def test_layer_level_methods_match_the_cpu_backend(hb, dtype, tol):
+    """compute_activation / train_step / train_finalize called on the layers themselves, the way code written
+    against the reference's layer classes does (_cpu_base_backend.py:44-68, 126-172; cpu_backend.py:13-52):
+    the same calls on both backends from the same seeded state, state compared after every call."""
+    from oracle import cpu_backend as ob
+    rng = np.random.default_rng(21)
+    n_pix, H, Mc, n_out, B = 40, 5, 12, 4, 24
+    x = synthetic_images(rng, B, n_pix).astype(dtype)
+    labels = one_hot_labels(rng, B, n_out).astype(dtype)
+    nets = [build_two_layer(b, 2 * n_pix, H, Mc, n_out, dict(MNIST_HP, l1_density=0.3), dtype, seed=5)
+            for b in (hb, ob)]
+    (g0, g1), (r0, r1) = nets[0]._layers, nets[1]._layers
+
+    def same(what):
+        for li, (gl, rl) in enumerate(((g0, r0), (g1, r1))):
+            for name in ("Ci", "Cj", "Cij", "weights", "bias") + (("kbi",) if li == 0 else ()):
+                e = rel_err(getattr(gl, name), getattr(rl, name), f"{what} L{li}.{name}", tol)
+                assert e <= tol, f"after {what}: L{li}.{name} {e:.3e}"
+        assert np.array_equal(g0.wmask, r0.wmask), what
+
+    for step, h in enumerate((None, 2, None, 0)):
+        ag, ar = g0.compute_activation(x), r0.compute_activation(x)
+        assert ag.shape == ar.shape and ag.dtype == dtype
+        assert rel_err(ag, ar, "hidden activation", tol) <= tol
+        g0.train_step(x, ar, h)  # both sides train on the same activation
+        r0.train_step(x, ar, h)
+        same(f"hidden train_step {step}")
+        bg, br = g1.compute_activation(ar), r1.compute_activation(ar)
+        assert rel_err(bg, br, "output activation", tol) <= tol
+        g1.train_step(ar, labels)
+        r1.train_step(ar, labels)
+        same(f"output train_step {step}")
+    g0.train_finalize(), r0.train_finalize(), g1.train_finalize(), r1.train_finalize()
+    same("train_finalize")
+    assert not np.array_equal(g0.wmask, build_two_layer(ob, 2 * n_pix, H, Mc, n_out, dict(MNIST_HP, l1_density=0.3),
+                                                        dtype, seed=5)._layers[0].wmask), "the calls rewired"
+    # a layer that has not joined a network says so
+    np.random.seed(1)
+    loose = hb.DenseLayer(8, 1, 3, 0.01, (0.1, 0.3, 0.03), dtype)
+    with pytest.raises(RuntimeError, match="add_layer"):
+        loose.compute_activation(np.zeros((2, 8), dtype))
+    with pytest.raises(TypeError):
+        g1.train_step(ar, labels, 0)
+
+
 def test_zero_period_schedule_does_not_rewire(hb):
     # 2 batches, 5 hypercolumns: 2 // 6 == 0.  The reference divides by zero here; this backend trains
     # without rewiring.
