@@ -48,6 +48,12 @@ struct Real<float> {
     return __builtin_amdgcn_logf(x) * 0.693147180559945309f;
   }
   static __device__ __forceinline__ float exp_(float x) { return expf(x); }
+  // exp for the softmax of the fused forward kernels, arguments <= 0: the hardware exp2 on x log2(e).  The
+  // product is rounded once, so the result is off by up to |x| 2^-24 relative -- below 1e-7 absolute for
+  // every x <= 0, which is what a softmax output is judged by.
+  static __device__ __forceinline__ float exp_nonpos(float x) {
+    return __builtin_amdgcn_exp2f(x * 1.44269504088896341f);
+  }
   // single IEEE operations: the pragma keeps the compiler from contracting them into FMAs
   static __device__ __forceinline__ float add(float a, float b) {
 #pragma clang fp contract(off)
@@ -77,6 +83,7 @@ struct Real<double> {
   static __device__ __forceinline__ double wlog_normal(double x) { return log(x); }
   static __device__ __forceinline__ double max_floor(double x, double floor) { return fmax(x, floor); }
   static __device__ __forceinline__ double exp_(double x) { return exp(x); }
+  static __device__ __forceinline__ double exp_nonpos(double x) { return exp(x); }
   static __device__ __forceinline__ double add(double a, double b) {
 #pragma clang fp contract(off)
     return a + b;

@@ -153,15 +153,21 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
     for (int t = 0; t < PT; t++) {
       const long col = lr + TPR * t;
       if (col < ncol) {
-        vals[t] = Real<T>::exp_(vals[t] - mx);
+        vals[t] = Real<T>::exp_nonpos(vals[t] - mx);
         sum += vals[t];
       }
     }
     sum = row16_reduce(sum, [](T x_, T y_) { return x_ + y_; });
 #pragma unroll
     for (int o = TPR / 2; o >= 16; o >>= 1) sum += __shfl_xor(sum, o);
+    if constexpr (sizeof(T) == 4) {  // one division per row, then products
+      const T r = T(1) / sum;
 #pragma unroll
-    for (int t = 0; t < PT; t++) vals[t] = vals[t] / sum;
+      for (int t = 0; t < PT; t++) vals[t] = vals[t] * r;
+    } else {
+#pragma unroll
+      for (int t = 0; t < PT; t++) vals[t] = vals[t] / sum;
+    }
   }
   if (b0 + row < B) {
     T *out = act + (b0 + row) * M + j0;
