@@ -667,6 +667,88 @@ def achievable_peaks():
     return 0
 
 
+def entry_point_rates(reps=200):
+    """The per-function entry points of the C ABI on device buffers at the headline layer's shape
+    (1568 -> 30 x 100, batch 128, mask density 0.1), each launched `reps` times back to back: time per
+    call and the rate on its algorithmic bytes or flops.  The network path uses the fused kernels; these
+    are what a caller that drives the reference's functions one by one gets."""
+    from streambrain_amd import _capi
+    from streambrain_amd._capi import DeviceArray
+    _capi.init(0)
+    lib, c = _capi.lib(), _capi.check
+    n, h, mc, b = 1568, 30, 100, 128
+    m = h * mc
+    rows = []
+    for dtype, sfx, R in ((np.float32, "_f32", ctypes.c_float), (np.float64, "_f64", ctypes.c_double)):
+        rng = np.random.default_rng(0)
+        es = np.dtype(dtype).itemsize
+        x = DeviceArray.from_numpy(rng.random((b, n)).astype(dtype))
+        act = DeviceArray.from_numpy(rng.random((b, m)).astype(dtype))
+        W = DeviceArray.from_numpy((0.1 * rng.standard_normal((n, m))).astype(dtype))
+        bias = DeviceArray.from_numpy(rng.random(m).astype(dtype))
+        kbi = DeviceArray.from_numpy(np.ones(m, dtype))
+        Ci = DeviceArray.from_numpy((0.05 + 0.1 * rng.random(n)).astype(dtype))
+        Cj = DeviceArray.from_numpy((0.005 + 0.01 * rng.random(m)).astype(dtype))
+        Cij = DeviceArray.from_numpy((0.001 * rng.random((n, m))).astype(dtype))
+        mask_host = (rng.random((n, h)) < 0.1).astype(np.uint8)
+        wmask = DeviceArray.from_numpy(mask_host)
+        pred = DeviceArray((b,), np.int32)
+        tau, cthr = 0.0001, 0.00005
+        masked_bytes = int((mask_host == 0).sum()) * mc * es + n * h
+        calls = [
+            ("sb_update_state", lambda: getattr(lib, "sb_update_state" + sfx)(act.ptr, x.ptr, W.ptr, bias.ptr, b, n, m),
+             None, 2.0 * b * n * m),
+            ("sb_softmax_minicolumns", lambda: getattr(lib, "sb_softmax_minicolumns" + sfx)(act.ptr, b, h, mc),
+             2 * b * m * es, None),
+            ("sb_compute_activation", lambda: getattr(lib, "sb_compute_activation" + sfx)(act.ptr, x.ptr, W.ptr, bias.ptr, b, n,
+                                                                               h, mc), None, 2.0 * b * n * m),
+            ("sb_add_bias", lambda: getattr(lib, "sb_add_bias" + sfx)(act.ptr, bias.ptr, b, m), 2 * b * m * es, None),
+            ("sb_update_weights", lambda: getattr(lib, "sb_update_weights" + sfx)(Ci.ptr, Cj.ptr, Cij.ptr, x.ptr, act.ptr,
+                                                                        R(tau), W.ptr, R(cthr), b, n, m),
+             3 * n * m * es, 2.0 * b * n * m),
+            ("sb_update_counters", lambda: getattr(lib, "sb_update_counters" + sfx)(Ci.ptr, Cj.ptr, Cij.ptr, x.ptr, act.ptr,
+                                                                          R(tau), b, n, m),
+             2 * n * m * es, 2.0 * b * n * m),
+            ("sb_weights_from_counters", lambda: getattr(lib, "sb_weights_from_counters" + sfx)(W.ptr, Ci.ptr, Cj.ptr, Cij.ptr,
+                                                                                      R(cthr), n, m),
+             2 * n * m * es, None),
+            ("sb_apply_mask", lambda: getattr(lib, "sb_apply_mask" + sfx)(W.ptr, wmask.ptr, n, h, mc), masked_bytes, None),
+            ("sb_update_bias_regularized",
+             lambda: getattr(lib, "sb_update_bias_regularized" + sfx)(bias.ptr, kbi.ptr, Cj.ptr, R(cthr), R(-500.0), R(0.3),
+                                                            R(0.0002), m), 4 * m * es, None),
+            ("sb_argmax_rows", lambda: getattr(lib, "sb_argmax_rows" + sfx)(act.ptr, b, m, pred.ptr), b * m * es, None),
+        ]
+        for name, call, nbytes, flops in calls:
+            for _ in range(10):
+                c(call())
+            best = float("inf")
+            for _ in range(3):
+                c(lib.sb_sync())
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    c(call())
+                c(lib.sb_sync())
+                best = min(best, (time.perf_counter() - t0) / reps)
+            row = {"entry_point": name + sfx, "us_per_call": round(1e6 * best, 2), "calls_timed": reps}
+            if nbytes is not None:
+                row["algorithmic_bytes"] = nbytes
+                row["GBps"] = round(nbytes / best / 1e9, 1)
+                row["frac_of_hbm_peak"] = round(nbytes / best / 1e9 / HBM_PEAK_GBS, 3)
+            if flops is not None:
+                peak = MFMA_PEAK_TFLOPS["f32" if es == 4 else "f64"]
+                row["flops"] = flops
+                row["TFLOPps"] = round(flops / best / 1e12, 2)
+                row["frac_of_mfma_peak"] = round(flops / best / 1e12 / peak, 3)
+            rows.append(row)
+        for d in (x, act, W, bias, kbi, Ci, Cj, Cij, wmask, pred):
+            d.free()
+    print(json.dumps({"entry_point_rates": {"shape": {"N": n, "H": h, "Mc": mc, "batch": b, "mask_density": 0.1},
+                                            "note": "back-to-back launches on the library's stream; a call of a few "
+                                                    "microseconds is bound by launch and completion (about 2.7 us)",
+                                            "rows": rows}}))
+    return 0
+
+
 def _pmc_medians(directory):
     import collections
     import csv
@@ -735,6 +817,8 @@ def main():
     ap.add_argument("--achievable-peaks", action="store_true",
                     help="only measure device-copy bandwidth and MFMA-only kernels (what the box reaches "
                          "next to the published peaks)")
+    ap.add_argument("--entry-point-rates", action="store_true",
+                    help="only time the per-function entry points of the C ABI at the headline layer's shape")
     ap.add_argument("--pmc-summary", metavar="DIR", help="summarise rocprofv3 --pmc csv output below DIR")
     ap.add_argument("--pmc-calibration", metavar="DIR",
                     help="with --pmc-summary: the same counters over `bench.py --copy-calibration`")
@@ -749,6 +833,8 @@ def main():
         return copy_calibration()
     if args.achievable_peaks:
         return achievable_peaks()
+    if args.entry_point_rates:
+        return entry_point_rates()
     if args.workload != "mnist":
         cfg = LARGE[args.workload]
         nb = (cfg["samples"] + cfg["batch"] - 1) // cfg["batch"]

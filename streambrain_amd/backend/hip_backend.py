@@ -36,6 +36,16 @@ except ImportError as exc:  # no fallback: the GPU module is the backend
 
 _backend.initialize(int(os.environ.get("BCPNN_HIP_DEVICE", "0")))
 
+# Progress bars as in the reference's fit (tqdm on rank 0), when tqdm is installed and BCPNN_HIP_PROGRESS is
+# not 0.  A bar costs one device synchronization per range of batches, _PROGRESS_RANGES per epoch.
+_PROGRESS_RANGES = 20
+_tqdm = None
+if os.environ.get("BCPNN_HIP_PROGRESS", "1") != "0":
+    try:
+        from tqdm import tqdm as _tqdm
+    except ImportError:
+        _tqdm = None
+
 
 _FLOAT_STATE = ("weights", "bias", "Ci", "Cj", "Cij")
 
@@ -188,10 +198,23 @@ class Network:
                 print('Layer - %d/%d' % (layer + 1, len(self._layers)), flush=True)
                 # the two draws of an epoch, in the reference's order (permutation(n) draws and returns what
                 # the reference's permutation(range(n)) does, without building the range element by element)
-                idx = np.random.permutation(n_samples)
-                hypercolumns_shuffled = np.random.permutation(self._layers[layer].hypercolumns)
-                self.net.train_epoch(layer, maximal_batch_size, idx.astype(np.int64),
-                                     hypercolumns_shuffled.astype(np.int64), epoch)
+                idx = np.random.permutation(n_samples).astype(np.int64)
+                hypercolumns_shuffled = np.random.permutation(self._layers[layer].hypercolumns).astype(np.int64)
+                if _tqdm is None:
+                    self.net.train_epoch(layer, maximal_batch_size, idx, hypercolumns_shuffled, epoch)
+                    continue
+                # the reference's per-batch progress bar (_cpu_base_backend.py:270-277, 311-312): the epoch is
+                # enqueued in ranges of batches and the bar advances when the device has finished a range
+                number_of_batches = (n_samples + maximal_batch_size - 1) // maximal_batch_size
+                per_range = max(1, number_of_batches // _PROGRESS_RANGES)
+                with _tqdm(total=number_of_batches) as pbar:
+                    pbar.set_description('Epoch %d/%d' % (epoch + 1, epochs))
+                    for first in range(0, number_of_batches, per_range):
+                        count = min(per_range, number_of_batches - first)
+                        self.net.train_batches(layer, maximal_batch_size, idx, hypercolumns_shuffled, epoch,
+                                               first, count, first + count == number_of_batches)
+                        self.net.synchronize()
+                        pbar.update(count)
         self.net.synchronize()
         self.net.training_done()
 

@@ -137,6 +137,24 @@ class PyNetwork {
     check(sb_net_train_epoch(net_, layer, (long)maximal_batch_size, sample_perm.data(), hc, epoch));
   }
 
+  // Batches [first_batch, first_batch + n_batches) of an epoch (sb_net_train_batches): what a caller
+  // that reports progress between ranges uses instead of train_epoch.
+  void train_batches(int layer, size_t maximal_batch_size, iarray sample_perm, py::object hc_perm, long epoch,
+                     long first_batch, long n_batches, bool finalize) {
+    if (sample_perm.ndim() != 1 || sample_perm.shape(0) != n_samples_)
+      throw std::runtime_error("train_batches: sample_perm must have one entry per training sample");
+    const int64_t *hc = nullptr;
+    iarray hc_arr;
+    if (!hc_perm.is_none()) {
+      hc_arr = iarray::ensure(hc_perm);
+      if (!hc_arr || hc_arr.ndim() != 1 || hc_arr.shape(0) != shape_of(layer).hypercolumns)
+        throw std::runtime_error("train_batches: hc_perm must have one entry per hypercolumn");
+      hc = hc_arr.data();
+    }
+    check(sb_net_train_batches(net_, layer, (long)maximal_batch_size, sample_perm.data(), hc, epoch, first_batch,
+                               n_batches, finalize ? 1 : 0));
+  }
+
   // The reference's signature: sample and hypercolumn orders come from this object's own generator
   // (time-seeded in the reference, dataloader.h:92 / helpers_random.h:12-23; see seed()).
   void train_layer(size_t maximal_batch_size, size_t layer, size_t epochs) {
@@ -238,6 +256,9 @@ void bind_network(py::module_ &m, const char *name) {
       .def("get_layer_state", &N::get_layer_state)
       .def("train_epoch", &N::train_epoch, py::arg("layer"), py::arg("maximal_batch_size"),
            py::arg("sample_perm"), py::arg("hc_perm"), py::arg("epoch"))
+      .def("train_batches", &N::train_batches, py::arg("layer"), py::arg("maximal_batch_size"),
+           py::arg("sample_perm"), py::arg("hc_perm"), py::arg("epoch"), py::arg("first_batch"),
+           py::arg("n_batches"), py::arg("finalize"))
       .def("evaluate_counts", &N::evaluate_counts)
       .def("forward", &N::forward)
       .def("layer_activation", &N::layer_activation)

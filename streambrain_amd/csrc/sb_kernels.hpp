@@ -86,6 +86,42 @@ __global__ __launch_bounds__(256) void k_weights_from_traces(T *W, const T *Ci, 
   }
 }
 
+// The same for M a multiple of VW and 16-byte aligned arrays: a thread owns VW consecutive columns (their
+// column reciprocals computed once) and walks kRowsPerTurn rows per turn with 16-byte accesses, all loads
+// of a turn in flight before the first is used.  Grid: x over blocks of 256 VW columns, y over row groups.
+constexpr int kRowsPerTurn = 8;
+template <typename T>
+__global__ __launch_bounds__(256) void k_weights_from_traces_vec(T *W, const T *Ci, const T *Cj, const T *Cij,
+                                                                 T cthr, T cthr4, long N, long M) {
+  constexpr int VW = Real<T>::VW;
+  using vec_t = typename Real<T>::vec_t;
+  const long j = ((long)blockIdx.x * 256 + threadIdx.x) * VW;
+  if (j >= M) return;
+  const vec_t cj = *reinterpret_cast<const vec_t *>(Cj + j);
+  T rcj[VW];
+#pragma unroll
+  for (int e = 0; e < VW; e++) rcj[e] = trace_reciprocal<T>(cj[e], cthr);
+  for (long i0 = (long)blockIdx.y * kRowsPerTurn; i0 < N; i0 += (long)gridDim.y * kRowsPerTurn) {
+    vec_t c[kRowsPerTurn];
+    T rci[kRowsPerTurn];
+#pragma unroll
+    for (int r = 0; r < kRowsPerTurn; r++) {
+      const long i = i0 + r < N ? i0 + r : N - 1;
+      c[r] = *reinterpret_cast<const vec_t *>(Cij + i * M + j);
+      rci[r] = Ci[i];
+    }
+#pragma unroll
+    for (int r = 0; r < kRowsPerTurn; r++) {
+      if (i0 + r >= N) break;
+      const T ri = trace_reciprocal<T>(rci[r], cthr);
+      vec_t w;
+#pragma unroll
+      for (int e = 0; e < VW; e++) w[e] = weight_from_traces<T>(c[r][e], ri, rcj[e], cthr4);
+      *reinterpret_cast<vec_t *>(W + (i0 + r) * M + j) = w;
+    }
+  }
+}
+
 // omp.cc:322-335.  A row of W per workgroup and turn; the hypercolumn of a column is a multiplication by a
 // constant the host prepares (M < 2^31).
 template <typename T>
@@ -96,6 +132,29 @@ __global__ __launch_bounds__(256) void k_apply_mask(T *W, const uint8_t *wmask, 
     const uint8_t *mrow = wmask + i * H;
     for (unsigned j = threadIdx.x; j < (unsigned)M; j += 256)
       if (mrow[by_Mc.div(j)] == 0) row[j] = T(0);
+  }
+}
+
+// The same for M and Mc multiples of VW and a 16-byte aligned W: a thread owns VW consecutive columns (one
+// hypercolumn) and stores 16-byte zero vectors; nothing of W is read.  Grid as k_weights_from_traces_vec.
+template <typename T>
+__global__ __launch_bounds__(256) void k_apply_mask_vec(T *W, const uint8_t *wmask, long N, long M, long H,
+                                                        FastDiv by_Mc) {
+  constexpr int VW = Real<T>::VW;
+  using vec_t = typename Real<T>::vec_t;
+  const long j = ((long)blockIdx.x * 256 + threadIdx.x) * VW;
+  if (j >= M) return;
+  const uint8_t *mcol = wmask + by_Mc.div((uint32_t)j);
+  vec_t zero;
+#pragma unroll
+  for (int e = 0; e < VW; e++) zero[e] = T(0);
+  for (long i0 = (long)blockIdx.y * kRowsPerTurn; i0 < N; i0 += (long)gridDim.y * kRowsPerTurn) {
+    uint8_t m[kRowsPerTurn];
+#pragma unroll
+    for (int r = 0; r < kRowsPerTurn; r++) m[r] = mcol[(i0 + r < N ? i0 + r : N - 1) * H];
+#pragma unroll
+    for (int r = 0; r < kRowsPerTurn; r++)
+      if (i0 + r < N && m[r] == 0) *reinterpret_cast<vec_t *>(W + (i0 + r) * M + j) = zero;
   }
 }
 
@@ -339,11 +398,18 @@ template <typename T>
 __device__ __forceinline__ long wave_argmax_first(const T *row, long M, int lane) {
   T best = T(0);
   long bi = -1;
-  for (long j = lane; j < M; j += 64) {
-    const T v = row[j];
-    if (bi < 0 || v > best) {
-      best = v;
-      bi = j;
+  constexpr int U = 8;  // loads in flight per lane before the (ordered) comparisons
+  for (long j0 = lane; j0 < M; j0 += 64 * U) {
+    T v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = row[j0 + 64 * u < M ? j0 + 64 * u : M - 1];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const long j = j0 + 64 * u;
+      if (j < M && (bi < 0 || v[u] > best)) {
+        best = v[u];
+        bi = j;
+      }
     }
   }
 #pragma unroll
@@ -443,6 +509,17 @@ template <typename T>
 __global__ __launch_bounds__(256) void k_fill(T *dst, T value, size_t n) {
   const size_t stride = (size_t)gridDim.x * 256;
   for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) dst[e] = value;
+}
+
+// Two short arrays copied in one launch (the new Ci and Cj of the per-function training entry points).
+template <typename T>
+__global__ __launch_bounds__(256) void k_copy_pair(T *dst1, const T *src1, size_t n1, T *dst2, const T *src2,
+                                                   size_t n2) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n1 + n2; e += stride) {
+    if (e < n1) dst1[e] = src1[e];
+    else dst2[e - n1] = src2[e - n1];
+  }
 }
 
 }  // namespace sb

@@ -132,6 +132,9 @@ template <typename T>
 int launch_mfma_probe(hipStream_t st, T *sink, long workgroups, long iters);
 template <typename T>
 int launch_fill(hipStream_t st, T *dst, T value, size_t n);
+// dst1[0 .. n1) = src1, dst2[0 .. n2) = src2 in one launch
+template <typename T>
+int launch_copy_pair(hipStream_t st, T *dst1, const T *src1, size_t n1, T *dst2, const T *src2, size_t n2);
 int launch_fill_bytes(hipStream_t st, void *dst, int value, size_t bytes);
 
 }  // namespace sb

@@ -315,6 +315,14 @@ int launch_weights_from_traces(hipStream_t st, T *W, const T *Ci, const T *Cj, c
   SB_REQUIRE(N > 0 && M > 0, "sizes must be positive");
   const TraceScalars<T> s = TraceScalars<T>::from(T(0), cthr);
   ProfScope prof_(st, K_APPLY_MASK);
+  constexpr int VW = Real<T>::VW;
+  if (M % VW == 0 && aligned16(W) && aligned16(Cij) && aligned16(Cj)) {
+    const long turns = cdiv(N, kRowsPerTurn);
+    hipLaunchKernelGGL((k_weights_from_traces_vec<T>), dim3((unsigned)cdiv(M, 256 * VW), (unsigned)(turns < 4096 ? turns : 4096)),
+                       dim3(256), 0, st, W, Ci, Cj, Cij, cthr, s.cthr4, N, M);
+    SB_LAUNCH_CHECK();
+    return 0;
+  }
   hipLaunchKernelGGL((k_weights_from_traces<T>), dim3((unsigned)(N < 8192 ? N : 8192)), dim3(256), 0, st, W, Ci,
                      Cj, Cij, cthr, s.cthr4, N, M);
   SB_LAUNCH_CHECK();
@@ -418,6 +426,14 @@ int launch_apply_mask(hipStream_t st, T *W, const uint8_t *wmask, long N, long H
   SB_REQUIRE(H * Mc < (1L << 31), "dimension too large");
   const long blocks = N < 8192 ? N : 8192;
   ProfScope prof_(st, K_APPLY_MASK);
+  constexpr int VW = Real<T>::VW;
+  if (Mc % VW == 0 && aligned16(W)) {
+    const long turns = cdiv(N, kRowsPerTurn);
+    hipLaunchKernelGGL((k_apply_mask_vec<T>), dim3((unsigned)cdiv(H * Mc, 256 * VW), (unsigned)(turns < 4096 ? turns : 4096)),
+                       dim3(256), 0, st, W, wmask, N, H * Mc, H, FastDiv::of(Mc));
+    SB_LAUNCH_CHECK();
+    return 0;
+  }
   hipLaunchKernelGGL((k_apply_mask<T>), dim3((unsigned)blocks), dim3(256), 0, st, W, wmask, N, H * Mc, H,
                      FastDiv::of(Mc));
   SB_LAUNCH_CHECK();
@@ -497,6 +513,17 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
   return 0;
 }
 
+template <typename T>
+int launch_copy_pair(hipStream_t st, T *dst1, const T *src1, size_t n1, T *dst2, const T *src2, size_t n2) {
+  if (n1 + n2 == 0) return 0;
+  SB_REQUIRE(dst1 && src1 && dst2 && src2, "null pointer");
+  const size_t blocks = (n1 + n2 + 255) / 256 < 4096 ? (n1 + n2 + 255) / 256 : 4096;
+  ProfScope prof_(st, K_FILL);
+  hipLaunchKernelGGL((k_copy_pair<T>), dim3((unsigned)blocks), dim3(256), 0, st, dst1, src1, n1, dst2, src2, n2);
+  SB_LAUNCH_CHECK();
+  return 0;
+}
+
 #define SB_INSTANTIATE_LAUNCHERS(T)                                                                   \
   template int launch_forward<T>(hipStream_t, T *, const T *, const T *, const T *, long, long, long, \
                                  long, bool);                                                         \
@@ -528,6 +555,7 @@ int launch_fill(hipStream_t st, T *dst, T value, size_t n) {
                                      unsigned long long *);                                           \
   template int launch_gather_rows<T>(hipStream_t, T *, const T *, const int64_t *, long, long);       \
   template int launch_mfma_probe<T>(hipStream_t, T *, long, long);                                    \
-  template int launch_fill<T>(hipStream_t, T *, T, size_t);
+  template int launch_fill<T>(hipStream_t, T *, T, size_t);                                           \
+  template int launch_copy_pair<T>(hipStream_t, T *, const T *, size_t, T *, const T *, size_t);
 
 }  // namespace sb

@@ -145,9 +145,7 @@ static int train_in_place(const T *x, const T *y, T *Cij, T *W, T *Ci, T *Cj, co
   rc = launch_train_fused<T>(st, x, y, Cij, W, Ci, Cj, ci_next, cj_next, wmask, bias_mode, bias, kbi, B,
                              N, H, Mc, taupdt, cthr, khalf, pmin, taubdt, false);
   if (rc) return rc;
-  SB_HIP(hipMemcpyAsync(Ci, ci_next, (size_t)N * sizeof(T), hipMemcpyDeviceToDevice, st));
-  SB_HIP(hipMemcpyAsync(Cj, cj_next, (size_t)M * sizeof(T), hipMemcpyDeviceToDevice, st));
-  return 0;
+  return launch_copy_pair<T>(st, Ci, ci_next, (size_t)N, Cj, cj_next, (size_t)M);
 }
 
 // ======================================================================================== network

@@ -183,7 +183,8 @@ def test_update_weights(k, oracle, dtype, B, N, M):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("B,N,M", [(5, 7, 9), (128, 257, 130), (96, 1568, 300), (33, 300, 10)])
+@pytest.mark.parametrize("B,N,M", [(5, 7, 9), (128, 257, 130), (96, 1568, 300), (33, 300, 10), (20, 37, 1032),
+                                   (16, 203, 3000)])
 def test_update_counters_then_weights(k, oracle, dtype, B, N, M):
     """The two halves of update_weights called one after the other (the cuda kernel set's form) give what
     the fused call gives: traces from update_counters, weights from update_weights(weights, Ci, Cj, Cij,
@@ -341,7 +342,7 @@ def test_update_mask_nan_scores(k, oracle, dtype, N):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("N,H,Mc", [(1, 1, 1), (13, 4, 5), (1568, 30, 100), (100, 7, 9)])
+@pytest.mark.parametrize("N,H,Mc", [(1, 1, 1), (13, 4, 5), (1568, 30, 100), (100, 7, 9), (37, 3, 260), (50, 40, 100)])
 def test_apply_mask(k, oracle, dtype, N, H, Mc):
     rng = np.random.default_rng(N)
     W = rng.standard_normal((N, H * Mc)).astype(dtype)

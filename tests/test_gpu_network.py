@@ -450,6 +450,26 @@ def test_zero_period_schedule_does_not_rewire(hb):
     assert np.all(np.isfinite(net._layers[0].weights))
 
 
+def test_progress_bar_changes_no_result(hb, monkeypatch):
+    """fit with the reference's per-batch progress bar enqueues an epoch in ranges of batches
+    (_cpu_base_backend.py:270-312); without tqdm it enqueues the epoch whole.  Same state either way,
+    over epochs with rewiring, a short last batch and both layers."""
+    rng = np.random.default_rng(8)
+    X, Y = synthetic_images(rng, 23 * 32 + 5, 60), one_hot_labels(rng, 23 * 32 + 5, 4)
+    states = []
+    for bar in (True, False):
+        if not bar:
+            monkeypatch.setattr(hb, "_tqdm", None)
+        assert (hb._tqdm is not None) == bar
+        net = build_two_layer(hb, 120, 4, 8, 4, MNIST_HP, np.float32, seed=2, density=0.3)
+        np.random.seed(11)
+        net.fit(X, Y, 32, [(0, 3), (1, 2)])
+        states.append([getattr(l, n) for l in net._layers for n in ("weights", "bias", "Ci", "Cj", "Cij")]
+                      + [net._layers[0].wmask, net._layers[0].kbi])
+    for a, b in zip(*states):
+        assert np.array_equal(a, b)
+
+
 def test_errors_are_python_exceptions(hb):
     net = hb.Network(np.float32)
     with pytest.raises(Exception):
