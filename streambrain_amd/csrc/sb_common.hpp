@@ -27,6 +27,13 @@ struct Real<float> {
   static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
   }
+  // Sixteen independent 4x4x1 products on one wavefront: block l/4 gets D[i][j] += A[i] * B[j] with A[i] from
+  // lane 4 (l/4) + i, B[j] from lane 4 (l/4) + j; D[i][j] is element i of lane 4 (l/4) + j's result.  With
+  // the operand registers of the 16x16x4 form (lane (p, q): row p, reduction index q) the blocks are
+  // (q, p / 4): rows 4 (p/4) .. +3 times 4 columns, one reduction index each; the four q are added afterwards.
+  static __device__ __forceinline__ acc_t mfma_4x4(float a, float b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, c, 0, 0, 0);
+  }
   static __device__ __forceinline__ int acc_row(int q, int v) { return 4 * q + v; }
   static __device__ __forceinline__ float log_(float x) { return logf(x); }
   // log for the weight recompute: the hardware log2 (1 ulp, v_log_f32) scaled by ln 2.  That

@@ -71,11 +71,15 @@ struct ForwardBias {
 // are summed through LDS in a fixed order (deterministic), then 16 threads per batch row add the bias
 // and, when FUSE, do the softmax over the tile's ncol columns.  bv: the thread's bias values
 // (ForwardBias::load).
-template <typename T, int NG, bool FUSE, int NWAVES, int LW>
+// tail: with TAIL, the tile's last four columns (tail_col0 .. +3 of the tile) as the 4x4 products of
+// Real<T>::mfma_4x4 leave them: element v of lane (p, q) is row 4 (p/4) + v, column p % 4, summed over the
+// reduction indices of q only.
+template <typename T, int NG, bool FUSE, int NWAVES, int LW, bool TAIL = false>
 __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&acc)[NG][Real<T>::VW],
                                                const T (&bv)[ForwardBias<T, NG, NWAVES>::PT],
                                                T (&red)[NWAVES / 2][16][TileCols<T, NG, LW>::CP], T *act,
-                                               long B, long M, long b0, long j0, long ncol) {
+                                               long B, long M, long b0, long j0, long ncol,
+                                               typename Real<T>::acc_t tail = {}) {
   using TC = TileCols<T, NG, LW>;
   constexpr int VW = Real<T>::VW;
   using vec_t = typename Real<T>::vec_t;
@@ -83,6 +87,15 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
   auto gcol = [](int g, int p_) { return TC::gcol(g, p_); };
   const int tid = threadIdx.x, lane = tid & 63, p = lane & 15, q = lane >> 4;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int tail_col0 = (NG - 1) * TC::GW + 16 * LW;
+  if constexpr (TAIL) {
+    static_assert(tail_col0 + 4 <= TC::CP, "tail columns inside the padded LDS row");
+#pragma unroll
+    for (int v = 0; v < 4; v++) {  // the four q in a fixed order
+      tail[v] += __shfl_xor(tail[v], 16);
+      tail[v] += __shfl_xor(tail[v], 32);
+    }
+  }
   // ---- cross-wavefront sum through LDS in a fixed order (deterministic): the upper half of the
   // wavefronts hands its partial tiles over, the lower half adds them to its own and publishes the
   // sums (each lane rewrites exactly the elements it has just read, so no barrier is needed between
@@ -105,6 +118,10 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
           for (int c = 0; c < LW; c++) slot[c] = acc[g][c][v];
         }
       }
+    if (TAIL && q == 0) {
+#pragma unroll
+      for (int v = 0; v < 4; v++) red[w - HALF][4 * (p >> 2) + v][tail_col0 + (p & 3)] = tail[v];
+    }
   }
   __syncthreads();
   if (w < HALF) {
@@ -123,6 +140,10 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
           for (int c = 0; c < LW; c++) slot[c] += acc[g][c][v];
         }
       }
+    if (TAIL && q == 0) {
+#pragma unroll
+      for (int v = 0; v < 4; v++) red[w][4 * (p >> 2) + v][tail_col0 + (p & 3)] += tail[v];
+    }
   }
   __syncthreads();
   // ---- bias (+ softmax): TPR threads per batch row, thread handles columns lr + TPR t
@@ -197,11 +218,18 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
 // RB: row blocks per workgroup.  The tile is 16*RB batch rows, every W vector a lane loads feeds RB MFMAs
 // instead of one, and W crosses the L2 -> L1 path 1/RB as often: for batches of many rows, where that path
 // is what bounds the kernel.  The epilogue handles the row blocks one after the other.
-template <typename T, int NG, bool FUSE, bool VEC, int NWAVES, int LW = Real<T>::VW, int RB = 1>
+//
+// TAIL (float): the hypercolumn ends with four columns beyond the last group's blocks (100 = 6 blocks of 16
+// + 4).  Instead of a seventh block, three quarters of it padding, they are multiplied as 4x4 products
+// (Real<T>::mfma_4x4) that take the x operand registers of the 16x16x4 form as they are and one extra
+// element of W per lane and step, at a quarter of a block's cost.
+template <typename T, int NG, bool FUSE, bool VEC, int NWAVES, int LW = Real<T>::VW, int RB = 1, bool TAIL = false>
 __global__ __launch_bounds__(64 * NWAVES) __attribute__((amdgpu_waves_per_eu(NWAVES / 4, NWAVES / 4)))
 void k_forward(ForwardArgs<T> a) {
   constexpr int VW = Real<T>::VW;
   static_assert(LW >= 1 && LW <= VW, "width of the last group");
+  static_assert(!TAIL || (sizeof(T) == 4 && FUSE && VEC), "the four-column tail: float, fused, vector loads");
+  constexpr int tail_col0 = (NG - 1) * 16 * VW + 16 * LW;  // first tail column of the tile
   auto gwidth = [](int g) { return g == NG - 1 ? LW : VW; };         // column blocks of group g
   auto gcol = [&](int g, int p_) { return g * (16 * VW) + gwidth(g) * p_; };  // first tile column of lane p_
   constexpr int GW = 16 * VW;
@@ -231,15 +259,19 @@ void k_forward(ForwardArgs<T> a) {
     for (int g = 0; g < NG; g++)
 #pragma unroll
       for (int c = 0; c < VW; c++) acc[r][g][c] = acc_t{0, 0, 0, 0};
+  acc_t tacc[RB];
+#pragma unroll
+  for (int r = 0; r < RB; r++) tacc[r] = acc_t{0, 0, 0, 0};
 
   // ring of D chunk buffers: D-1 chunks of loads are in flight while one is being multiplied
   constexpr int D = 2;  // measured: deeper rings are slower, the CU cannot keep more loads in flight anyway
   T xr[D][RB][VW];
   T wr[D][VW][NG][VW];
+  T wt[D][VW];  // TAIL: W[k, tail column p % 4] for the lane's VW reduction indices
 
-  auto compute = [&](const T(&xi)[RB][VW], const T(&wi)[VW][NG][VW]) {
+  auto compute = [&](const T(&xi)[RB][VW], const T(&wi)[VW][NG][VW], const T(&ti)[VW]) {
 #pragma unroll
-    for (int s = 0; s < VW; s++)
+    for (int s = 0; s < VW; s++) {
 #pragma unroll
       for (int g = 0; g < NG; g++)
 #pragma unroll
@@ -248,8 +280,13 @@ void k_forward(ForwardArgs<T> a) {
 #pragma unroll
             for (int r = 0; r < RB; r++) acc[r][g][c] = Real<T>::mfma(xi[r][s], wi[s][g][c], acc[r][g][c]);
           }
+      if constexpr (TAIL) {
+#pragma unroll
+        for (int r = 0; r < RB; r++) tacc[r] = Real<T>::mfma_4x4(xi[r][s], ti[s], tacc[r]);
+      }
+    }
   };
-  auto load_guarded = [&](long kc, T(&xo)[RB][VW], T(&wo)[VW][NG][VW]) {
+  auto load_guarded = [&](long kc, T(&xo)[RB][VW], T(&wo)[VW][NG][VW], T(&to)[VW]) {
     const long kk = kc * KC + VW * q;
 #pragma unroll
     for (int r = 0; r < RB; r++) {
@@ -272,6 +309,7 @@ void k_forward(ForwardArgs<T> a) {
           }
         }
       }
+      if constexpr (TAIL) to[s] = krow < a.N ? wrow[j0 + tail_col0 + (p & 3)] : T(0);
     }
   };
 
@@ -300,18 +338,26 @@ void k_forward(ForwardArgs<T> a) {
       for (int g = 0; g < NG; g++)
         wat[s][g] = j0 + gcol(g, p) < jend ? (unsigned)(((long)(VW * q + s) * a.M + gcol(g, p)) * ES)
                                            : BufferWindow<T>::kOutside;
+    unsigned tat[VW];  // TAIL
+#pragma unroll
+    for (int s = 0; s < VW; s++) tat[s] = (unsigned)(((long)(VW * q + s) * a.M + tail_col0 + (p & 3)) * ES);
     const long xstep = (long)NWAVES * KC;
     const long wstep = (long)NWAVES * KC * a.M;
     // Chunks w, w + NWAVES, ... < nfull: n of them for this wavefront.  The loop is branch-free: a load
     // past the last chunk reads whatever lies there (or zeros past the arrays) and is never used, so
     // the compiler can keep exact wait counts and D-1 chunks really are in flight.
     const long n = w < nfull ? (nfull - 1 - w) / NWAVES + 1 : 0;
-    auto load_next = [&](T(&xo)[RB][VW], T(&wo)[VW][NG][VW]) {
+    auto load_next = [&](T(&xo)[RB][VW], T(&wo)[VW][NG][VW], T(&to)[VW]) {
       const BufferWindow<T> xwin(xbase, xleft), wwin(wbase, wleft);
 #pragma unroll
       for (int r = 0; r < RB; r++) xwin.template load_n<VW>(xo[r], xat[r]);
 #pragma unroll
-      for (int s = 0; s < VW; s++)
+      for (int s = 0; s < VW; s++) {
+        if constexpr (TAIL) {
+          T one[1];
+          wwin.template load_n<1>(one, tat[s]);
+          to[s] = one[0];
+        }
 #pragma unroll
         for (int g = 0; g < NG; g++) {
           if (gwidth(g) == VW) {
@@ -323,12 +369,13 @@ void k_forward(ForwardArgs<T> a) {
             for (int e = 0; e < LW; e++) wo[s][g][e] = t[e];
           }
         }
+      }
       xbase += xstep, xleft -= xstep;
       wbase += wstep, wleft -= wstep;
     };
     if (n > 0) {
 #pragma unroll
-      for (int u = 0; u < D - 1; u++) load_next(xr[u], wr[u]);  // chunks 0 .. D-2
+      for (int u = 0; u < D - 1; u++) load_next(xr[u], wr[u], wt[u]);  // chunks 0 .. D-2
       __builtin_amdgcn_sched_barrier(0);
       long i = 0;
       for (; i + D <= n; i += D) {
@@ -336,26 +383,26 @@ void k_forward(ForwardArgs<T> a) {
         for (int u = 0; u < D; u++) {
           // the scheduling fences keep the loads where they are written: the compiler's latency model
           // would otherwise sink them to just ahead of their use, far too late for HBM or L2
-          load_next(xr[(u + D - 1) % D], wr[(u + D - 1) % D]);  // chunk i + u + D - 1
+          load_next(xr[(u + D - 1) % D], wr[(u + D - 1) % D], wt[(u + D - 1) % D]);  // chunk i + u + D - 1
           __builtin_amdgcn_sched_barrier(0);
-          compute(xr[u], wr[u]);                                              // chunk i + u
+          compute(xr[u], wr[u], wt[u]);                                       // chunk i + u
           __builtin_amdgcn_sched_barrier(0);
         }
       }
 #pragma unroll
       for (int u = 0; u < D - 1; u++)
-        if (i + u < n) compute(xr[u], wr[u]);
+        if (i + u < n) compute(xr[u], wr[u], wt[u]);
     }
     // partial last chunk (N % KC != 0): one wavefront takes it through the guarded path
     if (nfull * KC < a.N && w == (int)(nfull % NWAVES)) {
-      load_guarded(nfull, xr[0], wr[0]);
-      compute(xr[0], wr[0]);
+      load_guarded(nfull, xr[0], wr[0], wt[0]);
+      compute(xr[0], wr[0], wt[0]);
     }
   }
 #pragma unroll
   for (int r = 0; r < RB; r++) {
     if (r > 0) __syncthreads();  // the previous row block's sums have been read
-    forward_finish<T, NG, FUSE, NWAVES, LW>(acc[r], bv, red, a.act, a.B, a.M, b0 + 16 * r, j0, ncol);
+    forward_finish<T, NG, FUSE, NWAVES, LW, TAIL>(acc[r], bv, red, a.act, a.B, a.M, b0 + 16 * r, j0, ncol, tacc[r]);
   }
 }
 

@@ -156,6 +156,11 @@ __device__ __forceinline__ KeyIdx<uint32_t> wave_pick(KeyIdx<uint32_t> c) {
   return KeyIdx<uint32_t>{(uint32_t)(m >> 32), (int)(uint32_t)m - 1};
 }
 
+__device__ __forceinline__ void note_changed(int *changed, int *nchanged, int row) {
+  const int at = atomicAdd(nchanged, 1);
+  if (at < kMaxChangedRows) changed[at] = row;
+}
+
 template <typename T, int NT, int R>
 struct MaskSwapFast {
   using SK = ScoreKey<T>;
@@ -219,8 +224,9 @@ struct MaskSwapFast {
   }
 
   // true: the swaps are done and written back; false: nothing was changed, run the full scan
+  // changed / nchanged (LDS): the rows that end on the other side are appended there
   static __device__ bool run(const MaskArgs<T> &a, Shared &sh, const T (&score)[R], const int (&m)[R],
-                             const T (&nom)[R], const int (&cs)[R]) {
+                             const T (&nom)[R], const int (&cs)[R], int *changed, int *nchanged) {
     const int tid = threadIdx.x, lane = tid & 63;
     K key[R];
 #pragma unroll
@@ -324,6 +330,7 @@ struct MaskSwapFast {
     // the later row, as the sequential >= / <= scans do.  A row that changes sides takes the score of
     // its other side along (csum +- 1), computed once up front, so the loop holds no division.
     int nS = sh.ncand[0], nA = sh.ncand[1];
+    const int nS0 = nS, nA0 = nA;  // rows that change sides are appended from these slots on
     bool vS = lane < nS, vA = lane < nA;
     int iS = vS ? sh.cand[0][lane] : 0, iA = vA ? sh.cand[1][lane] : 0;
     int csS = vS ? sh.cand_cs[0][lane] : 0, csA = vA ? sh.cand_cs[1][lane] : 0;
@@ -357,14 +364,36 @@ struct MaskSwapFast {
     if (vS) {
       a.wmask[(long)iS * a.H + a.h] = 0;
       a.csum[iS] = csS;
+      if (lane >= nS0) note_changed(changed, nchanged, iS);
     }
     if (vA) {
       a.wmask[(long)iA * a.H + a.h] = 1;
       a.csum[iA] = csA;
+      if (lane >= nA0) note_changed(changed, nchanged, iA);
     }
     return true;
   }
 };
+
+// Steps 3 and 4 in the swap kernel's wake (a.W_fix != nullptr), by the whole workgroup: the weights of the
+// rows that changed sides -- every other row of the hypercolumn already holds what its unchanged mask byte
+// asks for -- and the hypercolumn's row list.  All threads of the workgroup call it.
+template <typename T, int NT>
+__device__ __forceinline__ void mask_swap_finish(const MaskArgs<T> &a, const int *changed, const int *nchanged) {
+  if (a.W_fix == nullptr) return;  // uniform
+  __syncthreads();                 // mask bytes and the list of changed rows are written
+  if (a.rows != nullptr) mask_rows_block<NT>(a.rows, a.row_cnt, a.wmask, a.N, a.H, a.cap, a.h);
+  const unsigned nc = *nchanged < kMaxChangedRows ? *nchanged : kMaxChangedRows, Mc = (unsigned)a.Mc;
+  for (unsigned e = threadIdx.x; e < nc * Mc; e += NT) {
+    const unsigned r = e / Mc, c = e - r * Mc;
+    const long i = changed[r], j = a.h * a.Mc + c;
+    T wgt = T(0);
+    if (a.wmask[i * a.H + a.h] != 0)
+      wgt = weight_from_traces<T>(a.Cij[i * a.M + j], trace_reciprocal<T>(a.Ci[i], a.cthr),
+                                  trace_reciprocal<T>(a.Cj[j], a.cthr), a.cthr4);
+    a.W_fix[i * a.M + j] = wgt;
+  }
+}
 
 // NT threads (64 to 1024 in powers of two), thread t owns rows t, t+NT, ..., t+(R-1)*NT.  1024 threads
 // with few rows each measured faster than 256 with more (1568 rows: 19.8 against 21.8 us).
@@ -373,7 +402,9 @@ __global__ __launch_bounds__(NT) void k_mask_swap_reg(MaskArgs<T> a) {
   constexpr int NWV = NT / 64;
   static_assert(NWV == 1 || NWV == 2 || NWV == 4 || NWV == 8 || NWV == 16, "1 to 16 wavefronts");
   __shared__ RowCand<T> part[2][4][NWV];  // [buffer][max0, min1, first0, first1][wavefront]
+  __shared__ int changed[kMaxChangedRows], nchanged;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  if (tid == 0) nchanged = 0;  // (published by the barrier below)
 
   T nom[R], score[R];
   int cs[R], m[R];  // m: 0 silent, 1 active, 2 not a candidate (row out of range or odd mask value)
@@ -400,7 +431,10 @@ __global__ __launch_bounds__(NT) void k_mask_swap_reg(MaskArgs<T> a) {
   const bool track_first = __syncthreads_or(has_nan) != 0;
   if (!track_first && a.iterations <= MaskSwapFast<T, NT, R>::TOPK) {
     __shared__ typename MaskSwapFast<T, NT, R>::Shared fast_lds;
-    if (MaskSwapFast<T, NT, R>::run(a, fast_lds, score, m, nom, cs)) return;
+    if (MaskSwapFast<T, NT, R>::run(a, fast_lds, score, m, nom, cs, changed, &nchanged)) {
+      mask_swap_finish<T, NT>(a, changed, &nchanged);
+      return;
+    }
     __syncthreads();
   }
 
@@ -494,8 +528,10 @@ __global__ __launch_bounds__(NT) void k_mask_swap_reg(MaskArgs<T> a) {
     if (dirty[k]) {
       a.wmask[i * a.H + a.h] = (uint8_t)m[k];
       a.csum[i] = cs[k];
+      note_changed(changed, &nchanged, (int)i);
     }
   }
+  mask_swap_finish<T, NT>(a, changed, &nchanged);
 }
 
 }  // namespace sb

@@ -196,7 +196,14 @@ struct MaskArgs {
   long N, M, H, Mc, h, iterations;
   T *nom;     // [N] scratch
   int *csum;  // [N] scratch
+  // Network path (k_mask_swap_reg only): after the swaps the same workgroup rewrites W[i, columns of h] of
+  // the rows that changed sides under the new mask (steps 3) and, with a row list, rebuilds the list of
+  // hypercolumn h (step 4).  W_fix == nullptr: neither.
+  T *W_fix;
+  int *rows, *row_cnt;
+  long cap;
 };
+constexpr int kMaxChangedRows = 64;  // rows that change sides in one merged launch: two per iteration
 
 template <typename T>
 __global__ __launch_bounds__(256) void k_mask_scores(MaskArgs<T> a) {
@@ -330,35 +337,45 @@ __global__ __launch_bounds__(1024) void k_mask_swap(MaskArgs<T> a) {
 
 // Step 4 (mask_rows_block / k_mask_rows): the list of connected rows of a hypercolumn, which the forward
 //   pass over connected rows walks:  rows[h * cap + 0 .. cnt_h) = ascending indices i with
-//   wmask[i, h] != 0, the rest of the cap entries -1; row_cnt[h] = cnt_h.  One workgroup of 256 threads
+//   wmask[i, h] != 0, the rest of the cap entries -1; row_cnt[h] = cnt_h.  One workgroup of NT threads
 //   per hypercolumn; entries beyond `cap` are dropped (the host sizes cap from the column counts, so
-//   none are).
+//   none are).  Each wavefront takes a contiguous run of rows, 64 at a time: a ballot gives a row's
+//   position among its 64, the wavefronts' totals meet in LDS (one barrier), and a second walk over the
+//   same mask bytes writes the entries.
+template <int NT = 256>
 __device__ __forceinline__ void mask_rows_block(int *rows, int *row_cnt, const uint8_t *wmask, long N, long H,
                                                 long cap, long h) {
-  __shared__ int scan[256];
-  const int tid = threadIdx.x;
-  const long seg = (N + 255) / 256;
-  const long lo = tid * seg < N ? tid * seg : N, hi = lo + seg < N ? lo + seg : N;
-  int mine = 0;
-  for (long i = lo; i < hi; i++) mine += wmask[i * H + h] != 0;
-  scan[tid] = mine;
+  constexpr int NWV = NT / 64;
+  __shared__ int wtot[NWV];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const long seg = ((N + NWV - 1) / NWV + 63) / 64 * 64;
+  const long lo = wv * seg, hi = lo + seg < N ? lo + seg : N;
+  int cnt = 0;
+  for (long i0 = lo; i0 < hi; i0 += 64) {
+    const long i = i0 + lane;
+    cnt += __popcll(__ballot(i < hi && wmask[i * H + h] != 0));
+  }
+  if (lane == 0) wtot[wv] = cnt;
   __syncthreads();
-  for (int o = 1; o < 256; o <<= 1) {  // inclusive scan of the per-thread counts
-    const int other = tid >= o ? scan[tid - o] : 0;
-    __syncthreads();
-    scan[tid] += other;
-    __syncthreads();
+  long pos = 0, total = 0;
+#pragma unroll
+  for (int u = 0; u < NWV; u++) {
+    const int t = wtot[u];
+    pos += u < wv ? t : 0;
+    total += t;
   }
   int *list = rows + h * cap;
-  long pos = scan[tid] - mine;
-  for (long i = lo; i < hi; i++)
-    if (wmask[i * H + h] != 0) {
-      if (pos < cap) list[pos] = (int)i;
-      pos++;
-    }
-  const long total = scan[255] < cap ? scan[255] : cap;
-  for (long k = total + tid; k < cap; k += 256) list[k] = -1;
-  if (tid == 0) row_cnt[h] = (int)total;
+  for (long i0 = lo; i0 < hi; i0 += 64) {
+    const long i = i0 + lane;
+    const bool on = i < hi && wmask[i * H + h] != 0;
+    const unsigned long long b = __ballot(on);
+    const long at = pos + __popcll(b & ((1ull << lane) - 1));
+    if (on && at < cap) list[at] = (int)i;
+    pos += __popcll(b);
+  }
+  if (total > cap) total = cap;
+  for (long k = total + threadIdx.x; k < cap; k += NT) list[k] = -1;
+  if (threadIdx.x == 0) row_cnt[h] = (int)total;
 }
 // hypercolumns h0 .. h0 + gridDim.x - 1  (a template only so that the header can be included from several
 // translation units)

@@ -107,6 +107,13 @@ template <typename T>
 int launch_update_mask(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, const T *Cj,
                        const T *Cij, T cthr, long N, long H, long Mc, long h, long iterations, T *nom,
                        int *csum);
+// The network's rewiring step: scores from the traces, the swaps, then W[:, columns of h] under the new mask
+// and (rows != nullptr) the row list of h -- in the swap kernel's wake where that kernel can, else through
+// launch_mask_fix_weights.
+template <typename T>
+int launch_rewire(hipStream_t st, uint8_t *wmask, T *W, const T *Ci, const T *Cj, const T *Cij, T cthr, long N,
+                  long H, long Mc, long h, long iterations, T *nom, int *csum, int *rows, int *row_cnt,
+                  long cap);
 // rows != nullptr: the row list of hypercolumn h (see launch_mask_rows) is rebuilt in the same launch.
 template <typename T>
 int launch_mask_fix_weights(hipStream_t st, T *W, const uint8_t *wmask, const T *Ci, const T *Cj,

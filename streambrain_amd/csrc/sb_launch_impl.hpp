@@ -118,6 +118,14 @@ int launch_forward_classify(hipStream_t st, T *act, const T *x, const T *W, cons
         SB_REQUIRE(grid < (1L << 31), "too many tiles for one launch");
         const dim3 g((unsigned)grid);
         if constexpr (sizeof(T) == 4) {
+          // 100 columns = 6 blocks of 16 + 4: the last four as 4x4 products instead of a seventh block
+          if (Mc == 6 * 16 + 4) {
+            if (rb == 4) hipLaunchKernelGGL((k_forward<T, 2, true, true, 8, 2, 4, true>), g, dim3(512), 0, st, a);
+            else if (rb == 2) hipLaunchKernelGGL((k_forward<T, 2, true, true, 8, 2, 2, true>), g, dim3(512), 0, st, a);
+            else hipLaunchKernelGGL((k_forward<T, 2, true, true, 8, 2, 1, true>), g, dim3(512), 0, st, a);
+            SB_LAUNCH_CHECK();
+            return 0;
+          }
           if (rb == 4) hipLaunchKernelGGL((k_forward<T, NGL, true, true, 8, LWL, 4>), g, dim3(512), 0, st, a);
         }
         if (rb == 4) {
@@ -365,10 +373,12 @@ int launch_update_bias_regularized(hipStream_t st, T *bias, T *kbi, const T *Cj,
 }
 
 // ---------------------------------------------------------------------------------------------- mask
+// W_fix != nullptr: the swap kernel also rewrites the weights of the rows that changed sides and (rows !=
+// nullptr) rebuilds the hypercolumn's row list, when it can (*merged = true); see MaskArgs.
 template <typename T>
-int launch_update_mask(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, const T *Cj,
-                       const T *Cij, T cthr, long N, long H, long Mc, long h, long iterations, T *nom,
-                       int *csum) {
+static int update_mask_impl(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, const T *Cj,
+                            const T *Cij, T cthr, long N, long H, long Mc, long h, long iterations, T *nom,
+                            int *csum, T *W_fix, int *rows, int *row_cnt, long cap, bool *merged) {
   SB_REQUIRE(wmask && Ci && Cj && Cij && nom && csum, "null pointer");
   SB_REQUIRE(N > 0 && H > 0 && Mc > 0, "sizes must be positive");
   SB_REQUIRE(h >= 0 && h < H, "hypercolumn index out of range");
@@ -379,6 +389,14 @@ int launch_update_mask(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, 
   a.wmask = wmask; a.W = W; a.Ci = Ci; a.Cj = Cj; a.Cij = Cij; a.cthr = cthr; a.cthr4 = s.cthr4;
   a.N = N; a.M = H * Mc; a.H = H; a.Mc = Mc; a.h = h; a.iterations = iterations; a.nom = nom;
   a.csum = csum;
+  // two rows change sides per iteration; the kernels for more than 65536 rows have no such tail
+  const bool merge = W_fix != nullptr && iterations > 0 && 2 * iterations <= kMaxChangedRows && N <= 65536 &&
+                     N * Mc < (1L << 31);
+  a.W_fix = merge ? W_fix : nullptr;
+  a.rows = merge ? rows : nullptr;
+  a.row_cnt = row_cnt;
+  a.cap = cap;
+  if (merged) *merged = merge;
   {
     ProfScope prof_(st, K_MASK_SCORES);
     hipLaunchKernelGGL((k_mask_scores<T>), dim3((unsigned)cdiv(N, 4)), dim3(256), 0, st, a);
@@ -399,6 +417,27 @@ int launch_update_mask(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, 
     SB_LAUNCH_CHECK();
   }
   return 0;
+}
+
+template <typename T>
+int launch_update_mask(hipStream_t st, uint8_t *wmask, const T *W, const T *Ci, const T *Cj,
+                       const T *Cij, T cthr, long N, long H, long Mc, long h, long iterations, T *nom,
+                       int *csum) {
+  return update_mask_impl<T>(st, wmask, W, Ci, Cj, Cij, cthr, N, H, Mc, h, iterations, nom, csum, nullptr,
+                             nullptr, nullptr, 0, nullptr);
+}
+
+template <typename T>
+int launch_rewire(hipStream_t st, uint8_t *wmask, T *W, const T *Ci, const T *Cj, const T *Cij, T cthr, long N,
+                  long H, long Mc, long h, long iterations, T *nom, int *csum, int *rows, int *row_cnt,
+                  long cap) {
+  SB_REQUIRE(W, "null pointer");
+  SB_REQUIRE(!rows || (row_cnt && cap > 0 && cap % 16 == 0), "row list arguments");
+  bool merged = false;
+  int rc = update_mask_impl<T>(st, wmask, (const T *)nullptr, Ci, Cj, Cij, cthr, N, H, Mc, h, iterations, nom,
+                               csum, W, rows, row_cnt, cap, &merged);
+  if (rc || merged) return rc;
+  return launch_mask_fix_weights<T>(st, W, wmask, Ci, Cj, Cij, cthr, N, H, Mc, h, rows, row_cnt, cap);
 }
 
 template <typename T>
@@ -548,6 +587,8 @@ int launch_copy_pair(hipStream_t st, T *dst1, const T *src1, size_t n1, T *dst2,
                                      const T *, T, long, long, long, long, long, T *, int *);         \
   template int launch_mask_fix_weights<T>(hipStream_t, T *, const uint8_t *, const T *, const T *,    \
                                           const T *, T, long, long, long, long, int *, int *, long);  \
+  template int launch_rewire<T>(hipStream_t, uint8_t *, T *, const T *, const T *, const T *, T, long, \
+                                long, long, long, long, T *, int *, int *, int *, long);              \
   template int launch_apply_mask<T>(hipStream_t, T *, const uint8_t *, long, long, long);             \
   template int launch_count_unmasked<T>(hipStream_t, const T *, const uint8_t *, long, long, long,    \
                                         unsigned long long *);                                        \

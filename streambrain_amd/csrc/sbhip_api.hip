@@ -315,12 +315,8 @@ static int layer_train_step(Layer &L, const T *x, const T *y, long B, long h) {
   // every entry of W has just been written under the mask
   if (L.plastic) L.w_masked = true, L.w_unchecked = false;
   if (L.plastic && h >= 0) {
-    rc = launch_update_mask<T>(st, L.wmask, (const T *)nullptr, (const T *)L.Ci, (const T *)L.Cj,
-                               (const T *)L.Cij, cthr, L.N, L.H, L.Mc, h, 16, (T *)L.nom, L.csum);
-    if (rc) return rc;
-    rc = launch_mask_fix_weights<T>(st, (T *)L.W, L.wmask, (const T *)L.Ci, (const T *)L.Cj,
-                                    (const T *)L.Cij, cthr, L.N, L.H, L.Mc, h, L.rows, L.row_cnt,
-                                    L.rows_cap);
+    rc = launch_rewire<T>(st, L.wmask, (T *)L.W, (const T *)L.Ci, (const T *)L.Cj, (const T *)L.Cij, cthr, L.N,
+                          L.H, L.Mc, h, 16, (T *)L.nom, L.csum, L.rows, L.row_cnt, L.rows_cap);
     // (a swap leaves the number of connected rows of the hypercolumn as it was, so its list still fits)
     if (rc) return rc;
   }
@@ -846,11 +842,8 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
                                khalf, pmin, taubdt);                                                   \
     if (rc || h < 0) return rc;                                                                        \
     if ((rc = ensure_mask_scratch(N))) return rc;                                                      \
-    rc = launch_update_mask<T>(g_ctx.stream, wmask, (const T *)nullptr, Ci, Cj, Cij, cthr, N, H, Mc,   \
-                               h, 16, (T *)g_ctx.mask_nom, g_ctx.mask_csum);                           \
-    if (rc) return rc;                                                                                 \
-    return launch_mask_fix_weights<T>(g_ctx.stream, W, wmask, Ci, Cj, Cij, cthr, N, H, Mc, h, nullptr, \
-                                      nullptr, 0);                                                     \
+    return launch_rewire<T>(g_ctx.stream, wmask, W, Ci, Cj, Cij, cthr, N, H, Mc, h, 16,                \
+                            (T *)g_ctx.mask_nom, g_ctx.mask_csum, nullptr, nullptr, 0);                \
   }
 
 SB_DEFINE_KERNEL_API(f32, float)
