@@ -362,7 +362,10 @@ def test_argmax_rows(k, oracle, dtype):
 # ------------------------------------------------------------------------ fused plastic train step
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("B,N,H,Mc,h", [(16, 40, 3, 8, None), (16, 40, 3, 8, 1), (128, 1568, 30, 100, None),
-                                        (128, 1568, 30, 100, 7), (96, 300, 4, 25, 3), (9, 33, 2, 7, 0)])
+                                        (128, 1568, 30, 100, 7), (96, 300, 4, 25, 3), (9, 33, 2, 7, 0),
+                                        # row counts of the wider swap kernels, whose launch also fixes the weights
+                                        # of the rows that changed sides, and past them (a separate fix-up launch)
+                                        (16, 3000, 3, 8, 2), (8, 9000, 2, 8, 0), (8, 65600, 2, 4, 1)])
 def test_plastic_train_step(k, oracle, dtype, B, N, H, Mc, h):
     _check_plastic_train_step(k, oracle, dtype, B, N, H, Mc, h, np.random.default_rng(B + N + H + Mc))
 
