@@ -156,6 +156,16 @@ __device__ __forceinline__ KeyIdx<uint32_t> wave_pick(KeyIdx<uint32_t> c) {
   return KeyIdx<uint32_t>{(uint32_t)(m >> 32), (int)(uint32_t)m - 1};
 }
 
+// Scatter inside a wavefront: v of every lane with `on` lands in lane `to`.  The targets must be distinct and
+// must be lanes that push themselves (a permutation among the pushing lanes); the other lanes keep 0.
+__device__ __forceinline__ uint32_t push_to_lane(uint32_t v, int to, bool on) {
+  const int lane = (int)(threadIdx.x & 63);
+  return (uint32_t)__builtin_amdgcn_ds_permute((on ? to : lane) * 4, on ? (int)v : 0);
+}
+__device__ __forceinline__ uint64_t push_to_lane(uint64_t v, int to, bool on) {
+  return ((uint64_t)push_to_lane((uint32_t)(v >> 32), to, on) << 32) | push_to_lane((uint32_t)v, to, on);
+}
+
 __device__ __forceinline__ void note_changed(int *changed, int *nchanged, int row) {
   const int at = atomicAdd(nchanged, 1);
   if (at < kMaxChangedRows) changed[at] = row;
@@ -338,6 +348,49 @@ struct MaskSwapFast {
     // keys as seen from the silent side (largest score wins) and from the active side (smallest wins)
     K kS = SK::of(mask_score<T>(nomS, csS)), kS_other = (K)~SK::of(mask_score<T>(nomS, csS + 1));
     K kA = (K)~SK::of(mask_score<T>(nomA, csA)), kA_other = SK::of(mask_score<T>(nomA, csA - 1));
+    // ---- All swaps at once, when that provably equals the loop below.  Rank the candidates of each side
+    // by (key, row index), the order the picks take them in; iteration k of the loop then picks the
+    // rank-k candidates of both sides and swaps them unless the silent one scores lower, so the number of
+    // swaps n is the length of the run of such pairs from rank 0 -- provided no row that changed sides
+    // is ever picked again.  That holds when every new active row scores strictly above, and every new
+    // silent row strictly below, the last pair the loop would look at; otherwise (blocks of equal scores,
+    // dead inputs) the loop runs.  Both sides must also hold a candidate for every iteration that happens.
+    {
+      const int kmax = (int)(a.iterations < (nS < nA ? nS : nA) ? a.iterations : (nS < nA ? nS : nA));
+      int rS = 0, rA = 0;
+      const int widest = nS > nA ? nS : nA;
+      for (int m = 0; m < widest; m++) {  // uniform
+        const K kSm = readlane_k(kS, m), kAm = readlane_k(kA, m);
+        const int iSm = __builtin_amdgcn_readlane(iS, m), iAm = __builtin_amdgcn_readlane(iA, m);
+        rS += (m < nS && (kSm > kS || (kSm == kS && iSm > iS))) ? 1 : 0;
+        rA += (m < nA && (kAm > kA || (kAm == kA && iAm > iA))) ? 1 : 0;
+      }
+      // lane k: the score keys of the rank-k silent and rank-k active candidates
+      const K sortedS = push_to_lane(kS, rS, vS), sortedA = (K)~push_to_lane(kA, rA, vA);
+      const unsigned long long keep_going = __ballot(lane < kmax && !(sortedS < sortedA));
+      const int n = __builtin_ctzll(~keep_going);  // (kmax <= 16: bit kmax is clear)
+      const bool complete = n < kmax || kmax == (int)a.iterations;
+      if (n == 0 && complete) return true;  // nothing to swap
+      if (complete) {
+        const int last = n < kmax ? n : kmax - 1;  // the last pair the loop looks at
+        const K lastS = readlane_k(sortedS, last), lastA = readlane_k(sortedA, last);
+        const bool toA = vS && rS < n, toS = vA && rA < n;
+        const bool again = (toA && !((K)~kS_other > lastA)) || (toS && !(kA_other < lastS));
+        if (__ballot(again) == 0) {
+          if (toA) {
+            a.wmask[(long)iS * a.H + a.h] = 1;
+            a.csum[iS] = csS + 1;
+            note_changed(changed, nchanged, iS);
+          }
+          if (toS) {
+            a.wmask[(long)iA * a.H + a.h] = 0;
+            a.csum[iA] = csA - 1;
+            note_changed(changed, nchanged, iA);
+          }
+          return true;
+        }
+      }
+    }
     for (long it = 0; it < a.iterations; it++) {
       KeyIdx<K> cmax{kS, vS ? iS : -1}, cmin{kA, vA ? iA : -1};
       cmax = wave_pick(cmax);
