@@ -470,6 +470,26 @@ def test_progress_bar_changes_no_result(hb, monkeypatch):
         assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_evaluate_of_many_batches_equals_single_batches(hb, dtype):
+    """evaluate / predict / forward over a set of many batches (uploaded in chunks of whole batches) give what
+    the same batches give when they are pushed through one at a time; the last batch is ragged."""
+    rng = np.random.default_rng(12)
+    n, B = 3000, 128
+    X, Y = synthetic_images(rng, n, 784), one_hot_labels(rng, n, 4)
+    net = build_two_layer(hb, 1568, 4, 8, 4, MNIST_HP, dtype, seed=5, density=0.3)
+    net.fit(X[:512], Y[:512], B, [(0, 2), (1, 1)])  # masked weights: the first layer walks row lists
+    whole = net.forward(X, B)
+    pred = net.predict(X, B)
+    correct, total = net.evaluate(X, Y, B)
+    assert whole.shape == (n, 4) and int(total[0]) == n
+    for lo in range(0, n, B):
+        part = net.forward(X[lo:lo + B], B)
+        assert np.array_equal(whole[lo:lo + B], part), lo
+    assert np.array_equal(pred, np.argmax(whole, axis=1))
+    assert int(correct[0]) == int((pred == np.argmax(Y, axis=1)).sum())
+
+
 def test_errors_are_python_exceptions(hb):
     net = hb.Network(np.float32)
     with pytest.raises(Exception):
