@@ -5,6 +5,7 @@
   python bench.py --workload dense|mnist15x200|wide64|stl10|largest    one of the other configurations alone
   python bench.py --achievable-peaks                                   device-copy and matrix-core probes
   python bench.py --copy-calibration                                   known-size copies for counter scaling
+  python bench.py --entry-point-rates                                  the per-function C entry points on their own
   python bench.py --pmc-summary DIR                                    text summary of rocprofv3 --pmc runs
 
 Headline workload: the MNIST-shaped 2-layer network, float32, batch 128, 60000 seeded
@@ -327,7 +328,10 @@ def headline(args):
 
     # Per-kernel durations: every launch of one more pass over the same number of steps is bracketed by
     # HIP events on the library's stream.
+    # (for a short window the bracketed pass runs on to about 200 steps in one go, so that a 20-step
+    # invocation does not price the kernels on 20 launches behind an idle gap)
     n_prof = min(args.steps, 2 * run.nb)
+    n_prof *= max(1, min(50, -(-200 // n_prof)))
     prof, raw_ms, brackets = run.profile(first, n_prof)
     bracket_us = calibrate_brackets(prof, raw_ms, brackets, dt * n_prof / args.steps)
 
