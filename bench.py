@@ -652,7 +652,7 @@ def achievable_peaks():
                               "frac_of_published_peak": 2 * nbytes / best / 1e9 / HBM_PEAK_GBS})
         src.free()
         dst.free()
-    for dtype, name in ((0, "f32"), (1, "f64")):
+    for dtype, name, shape in ((0, "f32", "16x16x4"), (1, "f64", "16x16x4"), (2, "f64", "4x4x4 (four blocks)")):
         flops = ctypes.c_double(0)
         c(lib.sb_probe_mfma(dtype, 2048, 1000, ctypes.byref(flops)))  # warm-up
         c(lib.sb_sync())
@@ -663,7 +663,7 @@ def achievable_peaks():
                 c(lib.sb_probe_mfma(dtype, 2048, iters, ctypes.byref(flops)))
                 c(lib.sb_sync())
                 best = min(best, time.perf_counter() - t0)
-            out["mfma"].append({"dtype": name, "instruction": "16x16x4", "workgroups": 2048, "what": what,
+            out["mfma"].append({"dtype": name, "instruction": shape, "workgroups": 2048, "what": what,
                                 "flops": flops.value, "ms": 1e3 * best, "TFLOPps": flops.value / best / 1e12,
                                 "published_peak_TFLOPps": MFMA_PEAK_TFLOPS[name],
                                 "frac_of_published_peak": flops.value / best / 1e12 / MFMA_PEAK_TFLOPS[name]})

@@ -289,10 +289,12 @@ const char *sb_profile_kernel_name(int kernel);
 int sb_profile_get(int kernel, double *total_ms, long *launches);
 
 /* Matrix-core probe for the achievable-peak record of bench.py: `workgroups` workgroups of four wavefronts
- * that issue nothing but 16x16x4 MFMAs of the given element type (8 * iters each); *flops receives the
- * launch's floating-point operations.  Stream-ordered; time it between sb_sync calls.  No counterpart in
- * the reference. */
-int sb_probe_mfma(int dtype /* sb_dtype */, long workgroups, long iters, double *flops);
+ * that issue nothing but 16x16x4 MFMAs of the given element type (8 * iters each), or, with
+ * SB_PROBE_F64_4X4X4, the 4x4x4 form of the fp64 MFMA (16 * iters each); *flops receives the launch's
+ * floating-point operations.  Stream-ordered; time it between sb_sync calls.  No counterpart in the
+ * reference. */
+#define SB_PROBE_F64_4X4X4 2
+int sb_probe_mfma(int dtype /* sb_dtype or SB_PROBE_F64_4X4X4 */, long workgroups, long iters, double *flops);
 
 #ifdef __cplusplus
 }

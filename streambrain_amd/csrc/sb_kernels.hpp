@@ -516,6 +516,25 @@ __global__ __launch_bounds__(256) void k_mfma_probe(T *sink, long iters) {
   if (s == T(-1)) sink[0] = s;  // never true: keeps the loop
 }
 
+// The same with the 4x4x4 form of the fp64 MFMA (four independent 4x4x4 products per instruction): sixteen
+// independent accumulators, 16 * iters instructions per wavefront.  On gfx950 this form issues at the
+// published fp64 matrix rate, the 16x16x4 form at two thirds of it.
+template <int UNUSED = 0>
+__global__ __launch_bounds__(256) void k_mfma_probe_f64_4x4x4(double *sink, long iters) {
+  double acc[16];
+#pragma unroll
+  for (int k = 0; k < 16; k++) acc[k] = (double)k;
+  const double a = 1.0 + threadIdx.x * 1e-6, b = 1.0 - threadIdx.x * 1e-6;
+  for (long i = 0; i < iters; i++) {
+#pragma unroll
+    for (int k = 0; k < 16; k++) acc[k] = __builtin_amdgcn_mfma_f64_4x4x4f64(a, b, acc[k], 0, 0, 0);
+  }
+  double s = 0;
+#pragma unroll
+  for (int k = 0; k < 16; k++) s += acc[k];
+  if (s == -1.0) sink[0] = s;  // never true: keeps the loop
+}
+
 template <int UNUSED = 0>
 __global__ __launch_bounds__(256) void k_fill_bytes(uint8_t *dst, uint8_t value, size_t bytes) {
   const size_t stride = (size_t)gridDim.x * 256;

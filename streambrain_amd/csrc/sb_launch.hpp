@@ -137,6 +137,8 @@ int launch_gather_rows_blocked(hipStream_t st, T *dst, T *plain, const T *src, c
 // `workgroups` workgroups of four wavefronts, each wavefront 8 * iters MFMAs of 2 * 16 * 16 * 4 flops.
 template <typename T>
 int launch_mfma_probe(hipStream_t st, T *sink, long workgroups, long iters);
+// the 4x4x4 form of the fp64 MFMA: 16 * iters instructions of 2 * 4 * 4 * 4 * 4 flops per wavefront
+int launch_mfma_probe_f64_4x4x4(hipStream_t st, double *sink, long workgroups, long iters);
 template <typename T>
 int launch_fill(hipStream_t st, T *dst, T value, size_t n);
 // dst1[0 .. n1) = src1, dst2[0 .. n2) = src2 in one launch

@@ -1040,9 +1040,15 @@ int sb_net_train_epoch(sb_net *net, int layer, long maximal_batch_size, const in
 // Matrix-core probe (see k_mfma_probe); *flops receives the floating-point operations of the launch.
 static int mfma_probe(int dtype, long workgroups, long iters, double *flops) {
   SB_READY();
-  SB_REQUIRE(dtype == SB_F32 || dtype == SB_F64, "dtype must be SB_F32 or SB_F64");
+  SB_REQUIRE(dtype == SB_F32 || dtype == SB_F64 || dtype == SB_PROBE_F64_4X4X4,
+             "dtype must be SB_F32, SB_F64 or SB_PROBE_F64_4X4X4");
   int rc = ensure_trace_scratch(1);
   if (rc) return rc;
+  if (dtype == SB_PROBE_F64_4X4X4) {
+    rc = launch_mfma_probe_f64_4x4x4(g_ctx.stream, (double *)g_ctx.trace_next, workgroups, iters);
+    if (!rc && flops) *flops = (double)workgroups * 4.0 * (double)iters * 16.0 * 2.0 * 4 * 4 * 4 * 4;
+    return rc;
+  }
   rc = dtype == SB_F32 ? launch_mfma_probe<float>(g_ctx.stream, (float *)g_ctx.trace_next, workgroups, iters)
                        : launch_mfma_probe<double>(g_ctx.stream, (double *)g_ctx.trace_next, workgroups, iters);
   if (!rc && flops) *flops = (double)workgroups * 4.0 * (double)iters * 8.0 * 2.0 * 16 * 16 * 4;
