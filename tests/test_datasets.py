@@ -78,3 +78,31 @@ def test_checkpoint_round_trip(tmp_path):
     wrong = build_two_layer(ob, 24, 2, 5, 3, MNIST_HP, np.float32, seed=2)
     with pytest.raises(ValueError):
         checkpoint.load_state(wrong, tmp_path / "state.npz")
+
+
+def test_example_driver_command_line_and_presets():
+    """The driver's presets are the reference's published hyper-parameters (train.py:71-139 there; a few
+    spot values), its command line rejects what the reference's rejects, and its synthetic data has the
+    dataset's shapes."""
+    import pytest
+    from streambrain_amd import train as driver
+
+    assert set(driver.PRESETS) == {"mnist", "fashion_mnist", "stl-10"}
+    m, f, s = (driver.PRESETS[k] for k in ("mnist", "fashion_mnist", "stl-10"))
+    assert (m.hypercolumns, f.hypercolumns, s.hypercolumns) == (15, 30, 15)
+    assert (m.epochs, f.epochs, s.epochs) == ((30, 60), (30, 60), (100, 20))
+    assert m.khalf == -139.02586632856327 and s.mask_iterations == 584 and s.n_inputs == 27648
+    assert f.classifier_taupdt == 0.00202951854188782 and s.unlabeled_rows == 15000
+    with pytest.raises(SystemExit):
+        driver.main(["cifar", "single", "128"])
+    with pytest.raises(SystemExit):
+        driver.main(["mnist", "half", "128"])
+    with pytest.raises(SystemExit):
+        driver.main(["mnist", "single", "128", "--epochs", "3"])
+    with pytest.raises(ValueError):
+        driver.run("mnist", np.float32, 0, synthetic=8)
+    hx, hy, tx, ty, ex, ey = driver.synthetic_data(s, 12, np.float64)
+    assert hx.shape == (12, 27648) and hy.shape == (12, 10) and not hy.any()
+    assert tx.shape == (12, 27648) and ty.sum() == 12 and ex.shape == (2, 27648) and ey.shape == (2, 10)
+    hx, hy, tx, ty, ex, ey = driver.synthetic_data(m, 12, np.float32)
+    assert hx is tx and hy is ty and hx.dtype == np.float32 and 0 <= hx.min() and hx.max() <= 1

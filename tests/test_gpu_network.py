@@ -656,3 +656,43 @@ def test_example_script_flow_through_the_package(tmp_path, monkeypatch):
     assert total == 320
     test_acc = correct / total
     assert train_acc > 0.5 and test_acc > 0.5, (train_acc, test_acc)
+
+
+def test_example_driver_on_files_and_synthetic_data(tmp_path, capsys):
+    """`python -m streambrain_amd.train` (the reference's train.py command line, train.py:44-215 there): on
+    idx-ubyte files written here with a learnable toy problem it trains, saves, and a second network loaded
+    from the file evaluates to the same counts; on synthetic data of the dataset's shape it runs through and
+    prints the reference's three result lines."""
+    from streambrain_amd import train as driver
+
+    rng = np.random.default_rng(5)
+
+    def write(name, header, payload):
+        with open(tmp_path / name, "wb") as f:
+            f.write(bytes(header))
+            f.write(payload.tobytes())
+
+    for split, n in (("train", 1536), ("t10k", 256)):
+        lab = rng.integers(0, 10, n).astype(np.uint8)
+        px = ((rng.random((n, 784)) < 0.03) * rng.integers(1, 120, (n, 784)))
+        for k in range(n):
+            px[k, 78 * int(lab[k]):78 * int(lab[k]) + 78] = rng.integers(150, 256, 78)
+        write(f"{split}-images-idx3-ubyte", [0, 0, 8, 3] + [0] * 12, px.astype(np.uint8))
+        write(f"{split}-labels-idx1-ubyte", [0, 0, 8, 1] + [0] * 4, lab)
+
+    state = tmp_path / "state.npz"
+    train_s, test_s, correct, total = driver.run("mnist", np.float32, 128, data_dir=str(tmp_path),
+                                                 epochs=(40, 80), save=str(state))
+    assert total == 256 and train_s > 0 and test_s > 0
+    assert correct / total > 0.3, correct  # (ten classes)
+    # the saved state, loaded into a fresh network and trained for no epoch, evaluates to the same counts
+    _, _, correct2, total2 = driver.run("mnist", np.float32, 128, data_dir=str(tmp_path), epochs=(0, 0),
+                                        load=str(state))
+    assert (correct2, total2) == (correct, total)
+
+    capsys.readouterr()
+    driver.main(["fashion_mnist", "double", "64", "--synthetic", "384", "--epochs", "1,1"])
+    out = capsys.readouterr().out
+    assert "Training duration: " in out and "Testing duration:  " in out and "Accuracy:          " in out
+    acc = float(out.split("Accuracy:")[1].split()[0])
+    assert 0.0 <= acc <= 1.0
