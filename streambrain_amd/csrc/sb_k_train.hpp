@@ -115,9 +115,11 @@ __global__ __launch_bounds__(256) void k_trace_sums(TrainArgs<T> a) {
 }
 
 // Wavefronts per SIMD the registers are budgeted for.  Doubles: four (the LDS slabs allow four workgroups
-// per CU; left alone the compiler takes more registers than that allows).  Floats need no limit.
-template <typename T>
-constexpr int train_waves_per_simd() { return sizeof(T) == 8 ? 4 : 1; }
+// per CU; left alone the compiler takes more registers than that allows).  Floats: five for the variant that
+// layers of whole vectors take (it fits 96 registers without spilling; left alone the compiler takes 100 and
+// loses the fifth workgroup), four for the others (which would spill at five).
+template <typename T, bool VEC, int MB>
+constexpr int train_waves_per_simd() { return sizeof(T) == 8 ? 4 : (VEC && MB == 1 ? 5 : 4); }
 
 // A raw byte window (for the mask bytes of a tile's rows): bounds-checked like BufferWindow.
 struct ByteWindow {
@@ -139,7 +141,7 @@ struct ByteWindow {
 // inside one hypercolumn), VW otherwise.
 // PRE: Ci_next and Cj_next already hold the new traces (k_trace_sums): no column sums here.
 template <typename T, int KCH, bool VEC, int MB, bool PRE = false>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(train_waves_per_simd<T>())))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(train_waves_per_simd<T, VEC, MB>())))
 void k_train_fused(TrainArgs<T> a) {
   using R = Real<T>;
   using acc_t = typename R::acc_t;
@@ -148,19 +150,19 @@ void k_train_fused(TrainArgs<T> a) {
   constexpr int TS = 64;                // tile side
   constexpr int G = TS / VW;            // 16-byte groups per slab row
   constexpr int RPP = 256 / G;          // slab rows the workgroup stages per pass
-  constexpr int SP = KCH / RPP;         // staging passes per chunk
+  constexpr int KC = KCH / 2;           // batch rows per chunk (two chunks' loads in flight, two slab buffers)
+  constexpr int SP = KC / RPP;          // staging passes per chunk
   constexpr int NG = 4 / VW;            // 16-byte vectors of a tile row held by one lane
   // The x slab has a pitch of 80 elements: lane (p, q) of wavefront w reads element 16 w + p of slab row
   // 4 s + q, and with a pitch of 64 the four q of a column would meet in one LDS bank.
   constexpr int XP = TS + 16;
   constexpr int SUMB = 8;               // LDS reads of the column sums in flight at a time
-  constexpr bool TILE_IN_LAST = sizeof(T) == 8;  // which chunk requests the Cij tile, see the chunk loop
   constexpr unsigned ES = sizeof(T);
   constexpr unsigned kOutside = BufferWindow<T>::kOutside;
-  static_assert(KCH % RPP == 0 && KCH % 4 == 0, "chunk size");
+  static_assert(KC % RPP == 0 && KC % 4 == 0, "chunk size");
 
-  __shared__ __attribute__((aligned(16))) T xs[KCH * XP];
-  __shared__ __attribute__((aligned(16))) T ys[KCH * TS];
+  __shared__ __attribute__((aligned(16))) T xs2[2][KC * XP];
+  __shared__ __attribute__((aligned(16))) T ys2[2][KC * TS];
   __shared__ __attribute__((aligned(16))) T rci_s[TS];
   __shared__ __attribute__((aligned(16))) T rcj_s[TS];
   __shared__ int slow_s[2];
@@ -203,26 +205,28 @@ void k_train_fused(TrainArgs<T> a) {
   const unsigned xat = i0 + VW * eg < N ? (er * N + i0 + VW * eg) * ES : kOutside;
   const unsigned yat = j0 + VW * eg < M ? (er * M + j0 + VW * eg) * ES : kOutside;
   const unsigned xstep = RPP * N * ES, ystep = RPP * M * ES;  // the next staging pass (uniform)
-  T sx[SP][VW], sy[SP][VW];
+  T sx[2][SP][VW], sy[2][SP][VW];  // two register sets: the loads of two chunks are in flight
   // Windows over the rows of one chunk: rows past the batch fall outside, and the per-lane offsets stay
   // those of chunk 0 whatever the batch size.  The chunk's first row advances by pointer; sizes are
   // 32-bit (KCH rows of x or y stay below 2 GiB).
   const T *xnext = a.x, *ynext = a.y;
   unsigned rows_left = (unsigned)a.B;  // B < 2^31 (launcher)
-  auto request_chunk = [&]() {
-    const unsigned rows = rows_left < (unsigned)KCH ? rows_left : (unsigned)KCH;
+  auto request_chunk = [&](auto set) {
+    constexpr int S = decltype(set)::value;
+    const unsigned rows = rows_left < (unsigned)KC ? rows_left : (unsigned)KC;
     const BufferWindow<T> xwin(xnext, typename BufferWindow<T>::Bytes{rows * N * ES}),
         ywin(ynext, typename BufferWindow<T>::Bytes{rows * M * ES});
 #pragma unroll
     for (int m = 0; m < SP; m++) {
-      xwin.load_vec(sx[m], xat, m * xstep);
-      ywin.load_vec(sy[m], yat, m * ystep);
+      xwin.load_vec(sx[S][m], xat, m * xstep);
+      ywin.load_vec(sy[S][m], yat, m * ystep);
     }
-    xnext += KCH * N;
-    ynext += KCH * M;
+    xnext += KC * N;
+    ynext += KC * M;
     rows_left -= rows;
   };
-  request_chunk();
+  request_chunk(std::integral_constant<int, 0>{});
+  request_chunk(std::integral_constant<int, 1>{});
 
   // ---- this lane's share of the tile, in the layout the MFMA leaves it in: wavefront w owns tile rows
   // 16 w .. 16 w + 15 and all 64 columns as four 16 x 16 blocks; the B operand of block c is column
@@ -315,24 +319,28 @@ void k_train_fused(TrainArgs<T> a) {
     if (odd) slow_s[role] = 1;
   };
 
-  // ---- chunks of the batch.  The loads of chunk c+1 are issued before chunk c is consumed from LDS,
-  // so their latency hides behind the MFMA loop and the column sums.
-  auto chunk = [&](long b0, auto with_tile) {
-    if (b0 > 0) __syncthreads();  // previous chunk fully consumed
+  // ---- chunks of the batch, KC rows each.  Chunk c is staged from register set c % 2 into slab buffer c % 2;
+  // the registers then take the loads of chunk c + 2, so two chunks are always on their way and a chunk's
+  // loads have two chunks' worth of MFMAs to arrive in.  One barrier per chunk: it publishes the slab, and
+  // since every wavefront reaches it only after its MFMA loop over the previous chunk, the buffer written in
+  // the next turn (read last two chunks ago) is free by then.
+  auto chunk = [&](auto set, auto with_tile, auto last) {
+    constexpr int S = decltype(set)::value;
+    T *xs = xs2[S], *ys = ys2[S];
 #pragma unroll
     for (int m = 0; m < SP; m++) {
       vec_t vx, vy;
 #pragma unroll
       for (int e = 0; e < VW; e++) {
-        vx[e] = sx[m][e];
-        vy[e] = sy[m][e];
+        vx[e] = sx[S][m][e];
+        vy[e] = sy[S][m][e];
       }
       *reinterpret_cast<vec_t *>(&xs[(er + RPP * m) * XP + VW * eg]) = vx;
       *reinterpret_cast<vec_t *>(&ys[(er + RPP * m) * TS + VW * eg]) = vy;
     }
-    __syncthreads();
-    request_chunk();  // the next one; past the batch: reads zeros nobody consumes
+    request_chunk(set);  // chunk c + 2; past the batch: reads zeros nobody consumes
     if (decltype(with_tile)::value) request_tile();
+    __syncthreads();
 
     if (!PRE && summer) {
       // Every addition below depends on the one before it.  Beside wavefronts that stream MFMAs such a chain
@@ -340,15 +348,15 @@ void k_train_fused(TrainArgs<T> a) {
       // the previous one retires queues behind the next MFMA on the SIMD's issue port), and at the default
       // priority it also queues behind the other wavefronts' vector work, while the rest of the workgroup
       // waits at the next barrier.  So in single precision the summing wavefronts run at the highest
-      // priority here, and above the others through their MFMA loop, in which they start late (measured at
-      // 1568 x 3000, batch 128: 17.2 -> 16.6 us per launch; in double precision, where an MFMA slot is three
-      // times as long, the same change costs 1 %, so the priorities stay as they are there).
+      // priority here, and above the others through their MFMA loop, in which they start late (in double
+      // precision, where an MFMA slot is three times as long, the same change costs 1 %, so the priorities
+      // stay as they are there).
       if constexpr (sizeof(T) == 4) __builtin_amdgcn_s_setprio(3);
       // rows past the end of the batch were staged as zeros: adding them changes nothing, so the loops
-      // need no guard; SUMB LDS reads are in flight before the (ordered) additions consume them
+      // need no guard; the LDS reads are in flight before the (ordered) additions consume them
       // (two copies so that the slab pitch is a constant and the reads take immediate offsets)
       if (sum_i) {
-        for (int r = 0; r < KCH; r += SUMB) {
+        for (int r = 0; r < KC; r += SUMB) {
           T v[SUMB];
 #pragma unroll
           for (int k = 0; k < SUMB; k++) v[k] = xs[(r + k) * XP + lane];
@@ -356,7 +364,7 @@ void k_train_fused(TrainArgs<T> a) {
           for (int k = 0; k < SUMB; k++) csum = R::add(csum, v[k]);
         }
       } else {
-        for (int r = 0; r < KCH; r += SUMB) {
+        for (int r = 0; r < KC; r += SUMB) {
           T v[SUMB];
 #pragma unroll
           for (int k = 0; k < SUMB; k++) v[k] = ys[(r + k) * TS + lane];
@@ -368,7 +376,7 @@ void k_train_fused(TrainArgs<T> a) {
 
     // after the last chunk's sums the new traces are complete: the two summing wavefronts turn them into
     // reciprocals for the weights while the others are still multiplying
-    if (summer && b0 + KCH >= a.B) finish_traces();
+    if (decltype(last)::value && summer) finish_traces();
     if constexpr (sizeof(T) == 4 && !PRE) {
       if (summer) __builtin_amdgcn_s_setprio(1);
     }
@@ -384,9 +392,9 @@ void k_train_fused(TrainArgs<T> a) {
 #pragma unroll
     for (int g = 0; g < NG; g++) yo[0][g] = *reinterpret_cast<const vec_t *>(ya + 16 * VW * g);
 #pragma unroll
-    for (int s = 0; s < KCH / 4; s++) {
+    for (int s = 0; s < KC / 4; s++) {
       const int cur = s & 1, nxt = cur ^ 1;
-      if (s + 1 < KCH / 4) {
+      if (s + 1 < KC / 4) {
         xo[nxt] = xa[(s + 1) * 4 * XP];
 #pragma unroll
         for (int g = 0; g < NG; g++)
@@ -398,17 +406,40 @@ void k_train_fused(TrainArgs<T> a) {
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  long b0 = 0;
-  if constexpr (TILE_IN_LAST) {
-    // doubles: a chunk takes twice as long, enough to cover the tile's latency, and the tile's registers
-    // then never coexist with the staging registers of a further chunk
-    for (; b0 + KCH < a.B; b0 += KCH) chunk(b0, std::false_type{});
-    chunk(b0, std::true_type{});
+  // Two chunks per turn, so that register sets and slab buffers have fixed names; a batch that is not a
+  // whole number of turns ends in a chunk of zeros.  The Cij tile (HBM latency) is requested late -- in
+  // single precision with three chunks left, in double precision, where a chunk takes twice as long and the
+  // tile's registers should not coexist with the staging registers of further chunks, with two -- and right
+  // after the loads of a chunk: loads return in issue order, so no chunk waits for the tile.  The turns from
+  // the request on are written out, so that every load sits in straight-line code (at a join the compiler
+  // would wait for all outstanding loads).
+  constexpr std::integral_constant<int, 0> set0{};
+  constexpr std::integral_constant<int, 1> set1{};
+  constexpr std::false_type no{};
+  constexpr std::true_type yes{};
+  const long turns = (a.B + 2 * KC - 1) / (2 * KC);
+  long t = 1;
+  if constexpr (sizeof(T) == 8) {
+    for (; t < turns; t++) {
+      chunk(set0, no, no);
+      chunk(set1, no, no);
+    }
+    chunk(set0, yes, no);
+    chunk(set1, no, yes);
   } else {
-    for (; b0 + 2 * KCH < a.B; b0 += KCH) chunk(b0, std::false_type{});
-    chunk(b0, std::true_type{});  // second-to-last (or only) chunk: the Cij tile is requested here
-    b0 += KCH;
-    if (b0 < a.B) chunk(b0, std::false_type{});
+    for (; t + 1 < turns; t++) {
+      chunk(set0, no, no);
+      chunk(set1, no, no);
+    }
+    if (turns >= 2) {
+      chunk(set0, no, no);
+      chunk(set1, yes, no);
+      chunk(set0, no, no);
+      chunk(set1, no, yes);
+    } else {
+      chunk(set0, yes, no);
+      chunk(set1, no, yes);
+    }
   }
 
   // ---- epilogue: decay + clamp and the Cij stores first (they need nothing from the other wavefronts),
