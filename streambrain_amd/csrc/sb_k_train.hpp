@@ -11,13 +11,15 @@
 // A workgroup (256 threads, 4 wavefronts) owns a 64 x 64 tile of Cij; 18 KiB of LDS and at most 96
 // registers per thread let five workgroups share a CU, so the 1175 tiles of a 1568 x 3000 layer are
 // all resident at once.
-//   1. Per chunk of KCH batch rows it stages x[:, i-tile] and y[:, j-tile] in LDS.  x and y are
+//   1. Per chunk of KCH / 2 batch rows it stages x[:, i-tile] and y[:, j-tile] in LDS.  x and y are
 //      "k-major" in memory, which is the 16x16x4 MFMA operand layout, so staging is a plain copy.  Each
 //      wavefront owns 16 rows x 64 columns of the tile (4 MFMA blocks) and feeds them with one element
 //      of x and one 16-byte vector of y per lane and K step of 4; the block columns are interleaved so
 //      that a lane's results of a row are consecutive columns, and the tile is loaded, updated and
 //      stored as 16-byte vectors straight from the accumulator registers (no pass through LDS).  The
-//      global loads of chunk c+1 are issued before chunk c is consumed.
+//      slabs are double-buffered and the global loads of two chunks are in flight: chunk c is staged from
+//      its registers, the registers take the loads of chunk c+2, and one barrier per chunk separates the
+//      staging from the MFMA loop.
 //   2. From the same LDS slabs, the lanes of one wavefront add up one column each of x, those of
 //      another one column each of y (which two wavefronts rotates with the tile index), in batch order
 //      b = 0..B-1 without FMA contraction: the reference's summation order, so Ci, Cj and kbi stay
@@ -26,9 +28,9 @@
 //      a tile column shares y: same inputs, same order, same bits).  The old traces are read from
 //      Ci/Cj and the new ones written to Ci_next/Cj_next by the tiles of the first tile column / row:
 //      no workgroup ever reads a value another one is writing.
-//   3. Global loads return in issue order, so the Cij tile (HBM latency) is requested only while the
-//      second-to-last chunk is being multiplied: the MFMA loop never waits for it, and it has arrived
-//      by the time the epilogue needs it.  All loads are branch-free (bounds-checked buffer windows
+//   3. Global loads return in issue order, so the Cij tile (HBM latency) is requested only with two or
+//      three chunks left, behind the loads of the last chunk: the MFMA loop never waits for it, and it has
+//      arrived by the time the epilogue needs it.  All loads are branch-free (bounds-checked buffer windows
 //      instead of guards): a guarded load makes the compiler wait for every outstanding load at the
 //      join.
 //   4. Epilogue per 16-byte vector: decay + clamp, weight, mask, one store each to Cij and W.  The
