@@ -293,8 +293,10 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   // row); loads are 16-byte accesses for every shape, and neither needs more than element alignment
   const bool vec = M % VW == 0;
   const dim3 grid((unsigned)(a.tiles_i * a.tiles_j));  // one workgroup per tile
-  // batch rows staged per chunk: 18 KiB of LDS per workgroup, so five workgroups share a CU
-  constexpr int KCH = 32;
+  // batch rows per turn of two chunks.  Floats: 32, 18 KiB of LDS per workgroup, so five workgroups share a
+  // CU.  Doubles: 16 -- the staging registers of two chunks of 8 rows leave the kernel without spills at four
+  // wavefronts per SIMD (1 % faster than 32 at 1568 x 10000, batch 512).
+  constexpr int KCH = sizeof(T) == 8 ? 16 : 32;
   const bool one_byte = Mc % VW == 0;  // every vector of VW columns lies inside one hypercolumn
   ProfScope prof_(st, K_TRAIN_FUSED);
   // Every tile adds up the batch's x and y columns for its own rows and columns, which with many tile
