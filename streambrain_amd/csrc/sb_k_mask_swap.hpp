@@ -210,7 +210,12 @@ struct MaskSwapFast {
     __syncthreads();
 #pragma unroll
     for (int g = 0; g < 2; g++) {
-      for (int w2 = wv + 1; w2 < NWV; w2++) incl[g] += sh.wtot[g][w2];
+      // (all totals requested at once; the ones of the wavefronts behind this one are added)
+#pragma unroll
+      for (int w2 = 0; w2 < NWV; w2++) {
+        const int v = sh.wtot[g][w2];
+        incl[g] += w2 > wv ? v : 0;
+      }
       const int after = incl[g] - c[g];
       if (active[g] && after < need[g] && need[g] <= incl[g]) {  // exactly one thread per group
         int acc = after;
