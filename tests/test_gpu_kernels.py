@@ -186,6 +186,26 @@ def test_update_weights(k, oracle, dtype, B, N, M):
 
 
 @pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("B", [1, 7, 8, 9, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 96, 100, 129])
+def test_fused_training_pass_at_batch_sizes_around_its_chunks(k, oracle, dtype, B):
+    """The fused kernel walks the batch two chunks of 16 (fp64: 8) rows per turn, the last turn padded with
+    zero rows, and requests the Cij tile a fixed number of chunks before the end: batch sizes on either side
+    of every boundary that schedule has (one turn, two turns, a half-filled last turn, a single row).
+    Traces bit for bit, Cij and W at the stated tolerance, W's zeros where the reference has them."""
+    rng = np.random.default_rng(1000 + B)
+    N, M = 131, 212
+    x, y, Ci, Cj, Cij = _trace_problem(rng, B, N, M, dtype)
+    tau = 0.01
+    cthr = tau / 2
+    r = oracle.update_weights(Ci.copy(), Cj.copy(), Cij.copy(), x, y, tau, np.zeros((N, M), dtype=dtype), cthr)
+    g = k.update_weights(Ci.copy(), Cj.copy(), Cij.copy(), x, y, tau, np.zeros((N, M), dtype=dtype), cthr)
+    assert np.array_equal(g[0], r[0]) and np.array_equal(g[1], r[1])
+    assert_close(g[2], r[2], dtype, "Cij")
+    assert_close(g[3], r[3], dtype, "W")
+    assert np.array_equal(g[3] == 0, r[3] == 0)
+
+
+@pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("B,N,M", [(5, 7, 9), (128, 257, 130), (96, 1568, 300), (33, 300, 10), (20, 37, 1032),
                                    (16, 203, 3000)])
 def test_update_counters_then_weights(k, oracle, dtype, B, N, M):
