@@ -167,8 +167,9 @@ def _trace_problem(rng, B, N, M, dtype):
                                            # batch of x above 2 MiB: tiles walked in panels of 8 tile
                                            # columns; 11 and 8 tile columns (narrow and no last panel)
                                            (64, 8300, 700), (48, 5600, 512),
-                                           # 150 x 141 tiles: the traces come from their own launch
-                                           (8, 9600, 9000)])
+                                           # 150 x 141 tiles: the traces come from their own launch (one
+                                           # turn of two chunks; two turns; a loop turn ahead of them)
+                                           (8, 9600, 9000), (40, 9600, 9000), (72, 7040, 6016)])
 def test_update_weights(k, oracle, dtype, B, N, M):
     rng = np.random.default_rng(B + 2 * N + 3 * M)
     x, y, Ci, Cj, Cij = _trace_problem(rng, B, N, M, dtype)
@@ -182,7 +183,11 @@ def test_update_weights(k, oracle, dtype, B, N, M):
     assert np.array_equal(g[1], r[1]), "Cj not bit-exact"
     assert_close(g[2], r[2], dtype, "Cij")
     assert_close(g[3], r[3], dtype, "W")
-    assert np.array_equal(g[3] == 0, r[3] == 0)
+    # zeros where the reference has zeros (dead rows and columns).  Among 86 million weights one or two
+    # have a logarithm argument within an ulp of 1, where one side's log gives exactly 0 and the other's
+    # a value of that last ulp: those are differences inside the tolerance, not of the zero pattern
+    differ = (g[3] == 0) != (r[3] == 0)
+    assert differ.sum() <= 4 and np.all(np.abs(g[3][differ]) + np.abs(r[3][differ]) <= 1e-6), differ.sum()
 
 
 @pytest.mark.parametrize("dtype", DT)
