@@ -194,8 +194,9 @@ int sb_net_create(sb_net **net, int dtype /* sb_dtype */);
 int sb_net_destroy(sb_net *net);
 
 /* PyNetwork::add_dense_layer (backend_full_cuda_internals.cu:653-665): counters start at the three
- * initial values; weights and bias start at zero until sb_net_set_layer_state is called.
- * Returns the layer index (>= 0) or a negative sb_status. */
+ * initial values; weights and bias start at zero and the mask of a plastic layer at all ones until
+ * sb_net_randomize_layer or sb_net_set_layer_state gives them values (a layer left at zero weights cannot
+ * learn: every softmax stays uniform).  Returns the layer index (>= 0) or a negative sb_status. */
 int sb_net_add_dense_layer(sb_net *net, long n_inputs, long hypercolumns, long minicolumns,
                            double taupdt, double initial_Ci, double initial_Cj,
                            double initial_Cij);
@@ -203,6 +204,13 @@ int sb_net_add_dense_layer(sb_net *net, long n_inputs, long hypercolumns, long m
 int sb_net_add_plastic_layer(sb_net *net, long n_inputs, long hypercolumns, long minicolumns,
                              double taupdt, double pmin, double khalf, double taubdt,
                              double initial_Ci, double initial_Cj, double initial_Cij);
+
+/* The initial state the reference's GPU backend object draws when a layer is constructed
+ * (backend_full_cuda_internals.cu:151-155: weights ~ N(0, 0.1), bias ~ 0.1 U(0, 1);
+ * helpers_training.cu:10-32: each mask byte of a plastic layer set with probability 0.1 -- `density`
+ * here), from a 64-bit Mersenne twister seeded with `seed`: the same seed gives the same state.  Drawn on
+ * the host and uploaded; synchronous.  sb_net_set_layer_state afterwards overrides any of it. */
+int sb_net_randomize_layer(sb_net *net, int layer, uint64_t seed, double density);
 
 /* State arrays of a layer, by name: "weights" [N,M], "bias" [M], "Ci" [N], "Cj" [M], "Cij" [N,M],
  * "kbi" [M] (plastic layers) in the network dtype, and "wmask" [N,H] uint8 (plastic layers).

@@ -53,6 +53,7 @@ _PLAIN_SIGS = {
     "sb_net_destroy": [_P],
     "sb_net_add_dense_layer": [_P, _L, _L, _L, _D, _D, _D, _D],
     "sb_net_add_plastic_layer": [_P, _L, _L, _L, _D, _D, _D, _D, _D, _D, _D],
+    "sb_net_randomize_layer": [_P, _I, ctypes.c_uint64, _D],
     "sb_net_set_layer_state": [_P, _I, ctypes.c_char_p, _P, _Z],
     "sb_net_get_layer_state": [_P, _I, ctypes.c_char_p, _P, _Z],
     "sb_net_set_training_data": [_P, _P, _P, _L, _L, _L],

@@ -178,10 +178,11 @@ class Network:
         if isinstance(layer, StructuralPlasticityLayer):
             index = self.net.add_plastic_layer(layer.in_features, layer.hypercolumns,
                                                layer.minicolumns, layer.taupdt, layer.pmin,
-                                               layer.khalf, layer.taubdt, cs[0], cs[1], cs[2])
+                                               layer.khalf, layer.taubdt, cs[0], cs[1], cs[2],
+                                               randomize=False)
         elif isinstance(layer, DenseLayer):
             index = self.net.add_dense_layer(layer.in_features, layer.hypercolumns, layer.minicolumns,
-                                             layer.taupdt, cs[0], cs[1], cs[2])
+                                             layer.taupdt, cs[0], cs[1], cs[2], randomize=False)
         else:
             raise Exception("Unknown layer type:", layer)
         layer._upload(self.net, index)

@@ -51,22 +51,30 @@ class PyNetwork {
     bool plastic;
   };
 
+  // Like the reference's object (backend_full_cuda_internals.cu:151-155, helpers_training.cu:10-32) a layer
+  // starts with random weights, bias and -- plastic layers -- a mask of density 0.1, here from this object's
+  // own generator (see seed()); `randomize = false` leaves them at zero / all ones for a caller that sets
+  // the state itself right away (set_layer_state).
+  static constexpr double kInitialDensity = 0.1;
+
   int add_dense_layer(size_t n_inputs, size_t n_hypercolumns, size_t n_minicolumns, double taupdt,
-                      double initial_Ci, double initial_Cj, double initial_Cij) {
+                      double initial_Ci, double initial_Cj, double initial_Cij, bool randomize) {
     int idx = sb_net_add_dense_layer(net_, (long)n_inputs, (long)n_hypercolumns, (long)n_minicolumns,
                                      taupdt, initial_Ci, initial_Cj, initial_Cij);
     check(idx);
     shapes_.push_back({(long)n_inputs, (long)n_hypercolumns, (long)n_minicolumns, false});
+    if (randomize) check(sb_net_randomize_layer(net_, idx, rng_(), kInitialDensity));
     return idx;
   }
 
   int add_plastic_layer(size_t n_inputs, size_t n_hypercolumns, size_t n_minicolumns, double taupdt,
                         double pmin, double khalf, double taubdt, double initial_Ci, double initial_Cj,
-                        double initial_Cij) {
+                        double initial_Cij, bool randomize) {
     int idx = sb_net_add_plastic_layer(net_, (long)n_inputs, (long)n_hypercolumns, (long)n_minicolumns,
                                        taupdt, pmin, khalf, taubdt, initial_Ci, initial_Cj, initial_Cij);
     check(idx);
     shapes_.push_back({(long)n_inputs, (long)n_hypercolumns, (long)n_minicolumns, true});
+    if (randomize) check(sb_net_randomize_layer(net_, idx, rng_(), kInitialDensity));
     return idx;
   }
 
@@ -246,8 +254,12 @@ void bind_network(py::module_ &m, const char *name) {
   using N = PyNetwork<REAL>;
   py::class_<N>(m, name)
       .def(py::init<>())
-      .def("add_dense_layer", &N::add_dense_layer)
-      .def("add_plastic_layer", &N::add_plastic_layer)
+      .def("add_dense_layer", &N::add_dense_layer, py::arg("n_inputs"), py::arg("n_hypercolumns"),
+           py::arg("n_minicolumns"), py::arg("taupdt"), py::arg("initial_Ci"), py::arg("initial_Cj"),
+           py::arg("initial_Cij"), py::arg("randomize") = true)
+      .def("add_plastic_layer", &N::add_plastic_layer, py::arg("n_inputs"), py::arg("n_hypercolumns"),
+           py::arg("n_minicolumns"), py::arg("taupdt"), py::arg("pmin"), py::arg("khalf"), py::arg("taubdt"),
+           py::arg("initial_Ci"), py::arg("initial_Cj"), py::arg("initial_Cij"), py::arg("randomize") = true)
       .def("initiate_training", &N::initiate_training)
       .def("train_layer", &N::train_layer)
       .def("training_done", &N::training_done)

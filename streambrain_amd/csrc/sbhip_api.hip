@@ -7,6 +7,7 @@
 #include <cstring>
 #include <utility>
 #include <mutex>
+#include <random>
 #include <string>
 #include <vector>
 
@@ -625,6 +626,36 @@ static int net_layer_train_step(sb_net *net, int layer, const void *h_in, const 
   return rc;
 }
 
+// Initial weights, bias and mask as the reference's GPU backend object draws them at construction
+// (backend_full_cuda_internals.cu:151-155: weights ~ N(0, 0.1), bias ~ 0.1 U(0, 1); helpers_training.cu:10-32:
+// mask bytes set with probability `density`, 0.1 there), from a generator seeded with `seed`.  Drawn on the
+// host in pieces of at most 64 MiB and uploaded; synchronous.
+template <typename T>
+static int net_randomize_layer(sb_net *net, int layer, uint64_t seed, double density) {
+  Layer &L = net->layers[layer];
+  std::mt19937_64 gen(seed);
+  std::normal_distribution<double> normal(0.0, 0.1);
+  std::uniform_real_distribution<double> uniform(0.0, 1.0);
+  const size_t nm = (size_t)L.N * L.M, piece = ((size_t)64 << 20) / sizeof(T);
+  std::vector<T> buf(std::min(nm, piece));
+  for (size_t lo = 0; lo < nm; lo += piece) {
+    const size_t n = std::min(piece, nm - lo);
+    for (size_t k = 0; k < n; k++) buf[k] = (T)normal(gen);
+    SB_HIP(hipMemcpy((T *)L.W + lo, buf.data(), n * sizeof(T), hipMemcpyHostToDevice));
+  }
+  buf.resize((size_t)L.M);
+  for (long j = 0; j < L.M; j++) buf[(size_t)j] = (T)(0.1 * uniform(gen));
+  SB_HIP(hipMemcpy(L.bias, buf.data(), (size_t)L.M * sizeof(T), hipMemcpyHostToDevice));
+  L.w_masked = false;
+  L.w_unchecked = true;
+  int rc = drop_frozen_cache(net);
+  if (rc || !L.plastic) return rc;
+  std::vector<uint8_t> mask((size_t)L.N * L.H);
+  for (auto &b : mask) b = uniform(gen) < density ? 1 : 0;
+  SB_HIP(hipMemcpy(L.wmask, mask.data(), mask.size(), hipMemcpyHostToDevice));
+  return layer_mask_replaced<T>(L, mask.data());
+}
+
 struct StateRef {
   void *ptr;
   size_t bytes;
@@ -981,6 +1012,16 @@ int sb_net_get_layer_state(sb_net *net, int layer, const char *name, void *h_dst
   SB_REQUIRE(h_dst, "null pointer");
   SB_REQUIRE(bytes == s.bytes, "size mismatch");
   return sb_memcpy_d2h(h_dst, s.ptr, bytes);
+}
+
+int sb_net_randomize_layer(sb_net *net, int layer, uint64_t seed, double density) {
+  SB_READY();
+  SB_REQUIRE(net, "null pointer");
+  SB_REQUIRE(layer >= 0 && layer < (int)net->layers.size(), "layer index out of range");
+  SB_REQUIRE(density >= 0.0, "density must be non-negative");
+  SB_HIP(hipStreamSynchronize(g_ctx.stream));
+  return net->dtype == SB_F32 ? net_randomize_layer<float>(net, layer, seed, density)
+                              : net_randomize_layer<double>(net, layer, seed, density);
 }
 
 int sb_net_set_training_data(sb_net *net, const void *h_images, const void *h_labels, long n_samples,

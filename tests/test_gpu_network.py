@@ -658,6 +658,79 @@ def test_example_script_flow_through_the_package(tmp_path, monkeypatch):
     assert train_acc > 0.5 and test_acc > 0.5, (train_acc, test_acc)
 
 
+@pytest.mark.parametrize("precision", [np.float32, np.float64])
+def test_backend_object_through_the_reference_methods_alone(precision):
+    """The C++ backend object driven the way the reference's full_cuda DSL drives its own
+    (full_cuda_backend/__init__.py:69-115 there): add_*_layer with the positional arguments, initiate_training,
+    train_layer, training_done, evaluate -> accuracy, and nothing else -- no state is handed in.  The object has
+    to bring a usable initial state of its own, as the reference's does (backend_full_cuda_internals.cu:151-155,
+    helpers_training.cu:10-32): random weights and bias and a mask of density 0.1.  On the learnable toy problem
+    of the example-script test: accuracy far above chance, hidden activations that are not uniform, and mask
+    columns that hold about a tenth of the inputs."""
+    import sys
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "streambrain_amd"))
+    import _bcpnn_backend_hip_internals as backend
+    backend.initialize(0)
+    rng = np.random.default_rng(3)
+
+    def make(n):
+        lab = rng.integers(0, 10, n)
+        px = (rng.random((n, 784)) < 0.03) * rng.integers(1, 120, (n, 784))
+        for k in range(n):
+            c = int(lab[k])
+            px[k, 78 * c:78 * c + 78] = rng.integers(150, 256, 78)
+        x = (px / 255.0).astype(precision)
+        return np.concatenate([x, 1 - x], axis=1), np.eye(10, dtype=precision)[lab]
+
+    train_x, train_y = make(1280)
+    test_x, test_y = make(320)
+    hp = MNIST_HP
+    H, Mc, N = 15, 20, 784 * 2
+    net = backend.PyNetwork_float32() if precision == np.float32 else backend.PyNetwork_float64()
+    net.seed(1234)  # (the reference seeds from the clock; a fixed seed keeps the test repeatable)
+    net.add_plastic_layer(N, H, Mc, hp["l1_taupdt"] * 4, hp["l1_pmin"], hp["l1_khalf"], hp["l1_taubdt"],
+                          1, 1 / Mc, 1 / Mc)
+    net.add_dense_layer(H * Mc, 1, 10, hp["l2_taupdt"] * 40, 1 / Mc, 1 / 10, 1 / (10 * Mc))
+
+    # the state the object drew for itself
+    W0, b0, mask0 = net.get_layer_state(0, "weights"), net.get_layer_state(0, "bias"), net.get_layer_state(0, "wmask")
+    assert abs(float(W0.std()) - 0.1) < 0.005 and abs(float(W0.mean())) < 0.002
+    assert 0 <= b0.min() and b0.max() <= 0.1 and b0.std() > 0.01
+    counts0 = mask0.sum(axis=0)
+    assert np.all(np.abs(counts0 - 0.1 * N) < 5 * np.sqrt(0.09 * N)), counts0
+    assert net.get_layer_state(1, "weights").std() > 0.05
+
+    net.initiate_training(train_x, train_y)
+    net.train_layer(64, 0, 4)  # 20 batches an epoch: with 15 hypercolumns, one rewiring per batch from epoch 1 on
+    net.train_layer(128, 1, 4)
+    net.training_done()
+    train_acc = net.evaluate(train_x, train_y, 128)
+    test_acc = net.evaluate(test_x, test_y, 128)
+    assert isinstance(train_acc, float) and 0.0 <= train_acc <= 1.0
+    assert train_acc > 0.5 and test_acc > 0.5, (train_acc, test_acc)  # chance: 0.1
+
+    # the hidden layer took sides: its softmax outputs are far from the uniform 1 / Mc
+    act = net.forward(test_x, 0, 128).reshape(-1, H, Mc)
+    assert np.allclose(act.sum(axis=2), 1, atol=1e-4 if precision == np.float32 else 1e-10)
+    assert float(act.max(axis=2).mean()) > 3.0 / Mc, float(act.max(axis=2).mean())
+    # rewiring swaps connections, so every mask column still holds what it was drawn with
+    mask = net.get_layer_state(0, "wmask")
+    assert np.array_equal(mask.sum(axis=0), counts0)
+    assert (mask != mask0).any(), "three epochs with rewiring moved no connection"
+    # weights are zero exactly under the mask (apply_mask)
+    W = net.get_layer_state(0, "weights")
+    assert np.all(W[np.repeat(mask, Mc, axis=1) == 0] == 0)
+
+    # two objects with the same seed draw the same state
+    a = backend.PyNetwork_float32()
+    b = backend.PyNetwork_float32()
+    for o in (a, b):
+        o.seed(7)
+        o.add_plastic_layer(64, 3, 4, 0.01, 0.3, -100, 0.01, 1, 0.25, 0.25)
+    for name in ("weights", "bias", "wmask"):
+        assert np.array_equal(a.get_layer_state(0, name), b.get_layer_state(0, name))
+
+
 def test_example_driver_on_files_and_synthetic_data(tmp_path, capsys):
     """`python -m streambrain_amd.train` (the reference's train.py command line, train.py:44-215 there): on
     idx-ubyte files written here with a learnable toy problem it trains, saves, and a second network loaded
