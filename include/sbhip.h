@@ -50,6 +50,11 @@ int sb_sync(void);
 /* The library's stream as a hipStream_t, for callers that time or order work with HIP events. */
 void *sb_stream(void);
 
+/* Number of allocating runtime calls (device and pinned host memory, events) the library has made so far
+ * in this process: a call that promises to allocate nothing leaves it unchanged.  No counterpart in the
+ * reference. */
+long sb_allocation_calls(void);
+
 /* ---- device memory for callers that have no HIP runtime of their own (ctypes tests, bench) --- */
 int sb_malloc(void **d_ptr, size_t bytes);
 int sb_free(void *d_ptr);
@@ -127,8 +132,9 @@ int sb_update_weights_f64(double *d_Ci, double *d_Cj, double *d_Cij, const doubl
                           const double *d_a_o, double taupdt, double *d_W, double cthr, long B,
                           long N, long M);
 
-/* sb_update_weights_f32 for callers that cannot call hipMalloc (code under HIP graph capture, tight
- * serving loops, harnesses that forbid allocation).  No counterpart in the reference.  Same arguments
+/* sb_update_weights_f32 for callers that cannot call hipMalloc (tight serving loops, harnesses that
+ * forbid allocation; the launches go to the library's own stream, so this is not something a caller's
+ * stream capture could record).  No counterpart in the reference.  Same arguments
  * and results as sb_update_weights_f32; the intermediate new Ci / Cj live in a static device array of
  * SB_NOALLOC_MAX_UNITS floats (1 MiB, held by every GPU the library runs on until the process ends)
  * instead of a buffer the library grows on demand, so the call allocates and frees nothing.  Returns
@@ -241,6 +247,13 @@ int sb_net_training_done(sb_net *net);
  * Asynchronous: returns once the epoch is enqueued. */
 int sb_net_train_epoch(sb_net *net, int layer, long maximal_batch_size,
                        const int64_t *h_sample_perm, const int64_t *h_hc_perm, long epoch_index);
+
+/* Upper bound, in bytes (both copies together), of the cache of frozen layers' activations that
+ * sb_net_train_epoch keeps while the last layer trains; 16 GiB unless set.  0 switches the cache off: every
+ * step then runs the forward passes of the layers below, as the reference does
+ * (_cpu_base_backend.py:279-295), with identical results.  A cache already held that exceeds the new bound
+ * is dropped. */
+int sb_net_set_frozen_cache_limit(sb_net *net, size_t bytes);
 
 /* A contiguous range of an epoch's batches [first_batch, first_batch + n_batches): sb_net_train_epoch
  * is the whole range with finalize = 1.  The sample order is applied when first_batch == 0 (it may be

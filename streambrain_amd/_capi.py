@@ -56,6 +56,7 @@ _PLAIN_SIGS = {
     "sb_net_randomize_layer": [_P, _I, ctypes.c_uint64, _D],
     "sb_net_set_layer_state": [_P, _I, ctypes.c_char_p, _P, _Z],
     "sb_net_get_layer_state": [_P, _I, ctypes.c_char_p, _P, _Z],
+    "sb_net_set_frozen_cache_limit": [_P, _Z],
     "sb_net_set_training_data": [_P, _P, _P, _L, _L, _L],
     "sb_net_training_done": [_P],
     "sb_net_train_epoch": [_P, _I, _L, _P, _P, _L],
@@ -73,7 +74,7 @@ _PLAIN_SIGS = {
     "sb_net_predict": [_P, _P, _L, _L, _L, _P],
     "sb_net_forward": [_P, _P, _L, _L, _I, _L, _P],
 }
-_RESTYPES = {"sb_last_error": ctypes.c_char_p, "sb_stream": _P}
+_RESTYPES = {"sb_last_error": ctypes.c_char_p, "sb_stream": _P, "sb_allocation_calls": _L}
 _OTHER_SIGS = {"sb_profile_kernel_name": ([_I], ctypes.c_char_p),
                "sb_profile_bracket_overhead_us": ([], _D)}
 

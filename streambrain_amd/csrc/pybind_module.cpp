@@ -180,6 +180,8 @@ class PyNetwork {
 
   void seed(uint64_t value) { rng_.seed(value); }
 
+  void set_frozen_cache_limit(size_t bytes) { check(sb_net_set_frozen_cache_limit(net_, bytes)); }
+
   void training_done() {
     check(sb_net_training_done(net_));
     n_samples_ = 0;
@@ -278,6 +280,7 @@ void bind_network(py::module_ &m, const char *name) {
       .def("layer_train_finalize", &N::layer_train_finalize)
       .def("predict", &N::predict)
       .def("seed", &N::seed)
+      .def("set_frozen_cache_limit", &N::set_frozen_cache_limit)
       .def("synchronize", &N::synchronize)
       .def("n_layers", &N::n_layers);
 }

@@ -261,7 +261,9 @@ void k_train_fused(TrainArgs<T> a) {
       for (int e = 0; e < MB; e++) {
         const unsigned hc = ecol[g] + e < M ? a.by_Mc.div(ecol[g] + e) : 0u;
 #pragma unroll
-        for (int v = 0; v < 4; v++) mb[v][g][e] = mwin.load(r0 * H + hc, v * rstep * H);
+        // (the row step goes into the per-lane offset, which the window's range check covers; the instruction's
+        // scalar offset is added after that check)
+        for (int v = 0; v < 4; v++) mb[v][g][e] = mwin.load((r0 + v * rstep) * H + hc, 0);
       }
   }
 
@@ -285,7 +287,15 @@ void k_train_fused(TrainArgs<T> a) {
 #pragma unroll
     for (int v = 0; v < 4; v++)
 #pragma unroll
-      for (int g = 0; g < NG; g++) cwin.load_vec(cpre[v][g], tat[g], v * vstep);
+      for (int g = 0; g < NG; g++) {
+        // A window of its own per row step, starting v row steps into the tile and shorter by as much: an
+        // instruction's scalar offset is added after the range check, so with the step passed there a lane whose
+        // first row is the tile's last would read rows past the tile (past the matrix, in the last tile row).
+        const unsigned skip = v * vstep;
+        const BufferWindow<T> win(a.Cij + (long)i0 * a.M + (long)v * rstep * a.M,
+                                  typename BufferWindow<T>::Bytes{tile_bytes > skip ? tile_bytes - skip : 0u});
+        win.load_vec(cpre[v][g], tat[g], 0);
+      }
   };
 
   acc_t acc[4];

@@ -24,6 +24,19 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line) {
   return SB_ERR_HIP;
 }
 
+// Every allocating runtime call of the library goes through these, so that a caller (and the test of the
+// entry point that promises to allocate nothing) can ask how many there have been: sb_allocation_calls.
+static long g_allocation_calls = 0;
+template <typename P>
+static hipError_t dev_malloc(P **p, size_t bytes) {
+  g_allocation_calls++;
+  return hipMalloc((void **)p, bytes);
+}
+static hipError_t event_create(hipEvent_t *e) {
+  g_allocation_calls++;
+  return hipEventCreate(e);
+}
+
 struct Context {
   bool ready = false;
   int device = 0;
@@ -72,7 +85,7 @@ static hipEvent_t prof_event() {
   if (!g_prof_pool.empty()) {
     e = g_prof_pool.back();
     g_prof_pool.pop_back();
-  } else if (hipEventCreate(&e) != hipSuccess) {
+  } else if (event_create(&e) != hipSuccess) {
     e = nullptr;
   }
   return e;
@@ -112,8 +125,8 @@ static int ensure_mask_scratch(long N) {
   g_ctx.mask_nom = nullptr;
   g_ctx.mask_csum = nullptr;
   g_ctx.mask_cap = 0;
-  SB_HIP(hipMalloc(&g_ctx.mask_nom, (size_t)N * sizeof(double)));
-  SB_HIP(hipMalloc((void **)&g_ctx.mask_csum, (size_t)N * sizeof(int)));
+  SB_HIP(dev_malloc(&g_ctx.mask_nom, (size_t)N * sizeof(double)));
+  SB_HIP(dev_malloc((void **)&g_ctx.mask_csum, (size_t)N * sizeof(int)));
   g_ctx.mask_cap = N;
   return 0;
 }
@@ -124,7 +137,7 @@ static int ensure_trace_scratch(long elems) {
   if (g_ctx.trace_next) SB_HIP(hipFree(g_ctx.trace_next));
   g_ctx.trace_next = nullptr;
   g_ctx.trace_cap = 0;
-  SB_HIP(hipMalloc(&g_ctx.trace_next, (size_t)elems * sizeof(double)));
+  SB_HIP(dev_malloc(&g_ctx.trace_next, (size_t)elems * sizeof(double)));
   g_ctx.trace_cap = elems;
   return 0;
 }
@@ -189,6 +202,7 @@ struct sb_net {
   // sample is computed once (Hc, data-set order) and shuffled per epoch like the images (Hcp).
   void *Hc = nullptr, *Hcp = nullptr;
   int Hc_layer = -1;  // Hc holds the activations of this layer for the current training set (-1: none)
+  size_t frozen_cache_limit = (size_t)16 << 30;  // bytes, both copies together (sb_net_set_frozen_cache_limit)
   unsigned long long *d_correct = nullptr;   // evaluate's counter
   unsigned long long *d_unmasked = nullptr;  // layer_check_masked's counter
 };
@@ -218,13 +232,13 @@ template <typename T>
 static int layer_alloc(Layer &L, T ci0, T cj0, T cij0) {
   hipStream_t st = g_ctx.stream;
   const size_t nm = (size_t)L.N * L.M;
-  SB_HIP(hipMalloc(&L.W, nm * sizeof(T)));
-  SB_HIP(hipMalloc(&L.Cij, nm * sizeof(T)));
-  SB_HIP(hipMalloc(&L.bias, L.M * sizeof(T)));
-  SB_HIP(hipMalloc(&L.Cj, L.M * sizeof(T)));
-  SB_HIP(hipMalloc(&L.Ci, L.N * sizeof(T)));
-  SB_HIP(hipMalloc(&L.Cj_alt, L.M * sizeof(T)));
-  SB_HIP(hipMalloc(&L.Ci_alt, L.N * sizeof(T)));
+  SB_HIP(dev_malloc(&L.W, nm * sizeof(T)));
+  SB_HIP(dev_malloc(&L.Cij, nm * sizeof(T)));
+  SB_HIP(dev_malloc(&L.bias, L.M * sizeof(T)));
+  SB_HIP(dev_malloc(&L.Cj, L.M * sizeof(T)));
+  SB_HIP(dev_malloc(&L.Ci, L.N * sizeof(T)));
+  SB_HIP(dev_malloc(&L.Cj_alt, L.M * sizeof(T)));
+  SB_HIP(dev_malloc(&L.Ci_alt, L.N * sizeof(T)));
   int rc = 0;
   if ((rc = launch_fill<T>(st, (T *)L.W, T(0), nm))) return rc;
   if ((rc = launch_fill<T>(st, (T *)L.Cij, cij0, nm))) return rc;
@@ -232,10 +246,10 @@ static int layer_alloc(Layer &L, T ci0, T cj0, T cij0) {
   if ((rc = launch_fill<T>(st, (T *)L.Cj, cj0, L.M))) return rc;
   if ((rc = launch_fill<T>(st, (T *)L.Ci, ci0, L.N))) return rc;
   if (L.plastic) {
-    SB_HIP(hipMalloc(&L.kbi, L.M * sizeof(T)));
-    SB_HIP(hipMalloc((void **)&L.wmask, (size_t)L.N * L.H));
-    SB_HIP(hipMalloc(&L.nom, L.N * sizeof(T)));
-    SB_HIP(hipMalloc((void **)&L.csum, L.N * sizeof(int)));
+    SB_HIP(dev_malloc(&L.kbi, L.M * sizeof(T)));
+    SB_HIP(dev_malloc((void **)&L.wmask, (size_t)L.N * L.H));
+    SB_HIP(dev_malloc(&L.nom, L.N * sizeof(T)));
+    SB_HIP(dev_malloc((void **)&L.csum, L.N * sizeof(int)));
     if ((rc = launch_fill<T>(st, (T *)L.kbi, T(1), L.M))) return rc;
     if ((rc = launch_fill_bytes(st, L.wmask, 1, (size_t)L.N * L.H))) return rc;
   }
@@ -260,7 +274,7 @@ static int ensure_act(sb_net *net, long rows) {
     SB_HIP(hipStreamSynchronize(g_ctx.stream));
     int rc = free_dev(L.act);
     if (rc) return rc;
-    SB_HIP(hipMalloc(&L.act, (size_t)rows * L.M * net->esize));
+    SB_HIP(dev_malloc(&L.act, (size_t)rows * L.M * net->esize));
     L.act_rows = rows;
   }
   return 0;
@@ -348,8 +362,8 @@ static int layer_mask_replaced(Layer &L, const uint8_t *mask) {
   }
   if (!sparse) return 0;
   if (!L.rows) {
-    SB_HIP(hipMalloc((void **)&L.rows, (size_t)L.H * cap * sizeof(int)));
-    SB_HIP(hipMalloc((void **)&L.row_cnt, (size_t)L.H * sizeof(int)));
+    SB_HIP(dev_malloc((void **)&L.rows, (size_t)L.H * cap * sizeof(int)));
+    SB_HIP(dev_malloc((void **)&L.row_cnt, (size_t)L.H * sizeof(int)));
     L.rows_cap = cap;
   }
   return launch_mask_rows(g_ctx.stream, L.rows, L.row_cnt, L.wmask, L.N, L.H, L.rows_cap, 0, L.H);
@@ -357,9 +371,8 @@ static int layer_mask_replaced(Layer &L, const uint8_t *mask) {
 
 // Largest cache of frozen activations kept (bytes, both copies together): at most 16 GiB, and at most half of
 // the device memory that is free when the cache is built; beyond it the activations are recomputed.
-static const size_t kFrozenCacheLimit = (size_t)16 << 30;
-static bool frozen_cache_affordable(size_t bytes) {
-  if (bytes > kFrozenCacheLimit) return false;
+static bool frozen_cache_affordable(const sb_net *net, size_t bytes) {
+  if (bytes > net->frozen_cache_limit) return false;
   size_t free_b = 0, total_b = 0;
   if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) {
     (void)hipGetLastError();
@@ -387,8 +400,8 @@ static int build_frozen_cache(sb_net *net, int upto, long maxB) {
   int rc = drop_frozen_cache(net);
   if (rc) return rc;
   // without the memory for both copies the caller goes on uncached (Hc_layer stays -1): not an error
-  if (hipMalloc(&net->Hc, (size_t)Ns * Mo * sizeof(T)) != hipSuccess ||
-      hipMalloc(&net->Hcp, (size_t)Ns * Mo * sizeof(T)) != hipSuccess) {
+  if (dev_malloc(&net->Hc, (size_t)Ns * Mo * sizeof(T)) != hipSuccess ||
+      dev_malloc(&net->Hcp, (size_t)Ns * Mo * sizeof(T)) != hipSuccess) {
     (void)hipGetLastError();
     net->Hcp = nullptr;
     if (net->Hc) (void)hipFree(net->Hc);
@@ -433,15 +446,15 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
   if (!last && (rc = drop_frozen_cache(net))) return rc;
   const long Mprev = layer > 0 ? net->layers[layer - 1].M : 0;
   const bool cache_fits = last && layer > 0 &&
-                          (net->Hc_layer == layer - 1 || frozen_cache_affordable(2 * (size_t)Ns * Mprev * sizeof(T)));
+                          (net->Hc_layer == layer - 1 || frozen_cache_affordable(net, 2 * (size_t)Ns * Mprev * sizeof(T)));
   if (permute) {
     SB_REQUIRE(h_sample_perm, "sample order missing");
     for (long r = 0; r < Ns; r++)
       SB_REQUIRE(h_sample_perm[r] >= 0 && h_sample_perm[r] < Ns, "sample index out of range");
 
     // images[idx, :] / labels[idx, :]  (_cpu_base_backend.py:258-260)
-    if (!net->Xp) SB_HIP(hipMalloc(&net->Xp, (size_t)Ns * net->NF * net->esize));
-    if (last && !net->Yp) SB_HIP(hipMalloc(&net->Yp, (size_t)Ns * net->NC * net->esize));
+    if (!net->Xp) SB_HIP(dev_malloc(&net->Xp, (size_t)Ns * net->NF * net->esize));
+    if (last && !net->Yp) SB_HIP(dev_malloc(&net->Yp, (size_t)Ns * net->NC * net->esize));
     SB_HIP(hipEventSynchronize(net->perm_copied));  // staging buffer free again
     std::memcpy(net->h_perm, h_sample_perm, (size_t)Ns * sizeof(int64_t));
     SB_HIP(hipMemcpyAsync(net->d_perm, net->h_perm, (size_t)Ns * sizeof(int64_t), hipMemcpyHostToDevice,
@@ -451,7 +464,7 @@ static int net_train_batches(sb_net *net, int layer, long maxB, const int64_t *h
     // second time, in blocks of 16 rows (batches must then start on block boundaries); one kernel writes
     // both copies from one read.
     if (net->layers[0].rows && maxB % 16 == 0) {
-      if (!net->XpB) SB_HIP(hipMalloc(&net->XpB, (size_t)cdiv_l(Ns, 16) * 16 * net->NF * net->esize));
+      if (!net->XpB) SB_HIP(dev_malloc(&net->XpB, (size_t)cdiv_l(Ns, 16) * 16 * net->NF * net->esize));
       if ((rc = launch_gather_rows_blocked<T>(st, (T *)net->XpB, (T *)net->Xp, (const T *)net->X, net->d_perm, Ns,
                                               net->NF)))
         return rc;
@@ -536,12 +549,12 @@ static int net_forward_batches(sb_net *net, const void *h_images, const void *h_
   if (chunk < maxB) chunk = maxB;
   if (chunk > n) chunk = n;
   ScopedDeviceBuffer bX, bY, bXB, bP;
-  SB_HIP(hipMalloc(&bX.p, (size_t)chunk * NF * sizeof(T)));
+  SB_HIP(dev_malloc(&bX.p, (size_t)chunk * NF * sizeof(T)));
   // a first layer that walks row lists also gets every chunk in blocks of 16 rows (see net_train_batches)
   const bool blocked = net->layers[0].rows && maxB % 16 == 0;
-  if (blocked) SB_HIP(hipMalloc(&bXB.p, (size_t)cdiv_l(chunk, 16) * 16 * NF * sizeof(T)));
-  if (h_labels) SB_HIP(hipMalloc(&bY.p, (size_t)chunk * NC * sizeof(T)));
-  if (h_pred) SB_HIP(hipMalloc(&bP.p, (size_t)chunk * sizeof(int32_t)));
+  if (blocked) SB_HIP(dev_malloc(&bXB.p, (size_t)cdiv_l(chunk, 16) * 16 * NF * sizeof(T)));
+  if (h_labels) SB_HIP(dev_malloc(&bY.p, (size_t)chunk * NC * sizeof(T)));
+  if (h_pred) SB_HIP(dev_malloc(&bP.p, (size_t)chunk * sizeof(int32_t)));
   void *const dX = bX.p, *const dY = bY.p, *const dXB = bXB.p;
   int32_t *const dP = (int32_t *)bP.p;
   if (h_labels) {
@@ -601,7 +614,7 @@ static int net_layer_activation(sb_net *net, int layer, const void *h_in, long r
   int rc = ensure_act(net, rows);
   if (rc) return rc;
   ScopedDeviceBuffer bX;
-  SB_HIP(hipMalloc(&bX.p, (size_t)rows * L.N * sizeof(T)));
+  SB_HIP(dev_malloc(&bX.p, (size_t)rows * L.N * sizeof(T)));
   SB_HIP(hipMemcpy(bX.p, h_in, (size_t)rows * L.N * sizeof(T), hipMemcpyHostToDevice));
   rc = layer_forward<T>(net, L, (const T *)bX.p, rows);
   if (!rc) SB_HIP(hipMemcpyAsync(h_act, L.act, (size_t)rows * L.M * sizeof(T), hipMemcpyDeviceToHost, g_ctx.stream));
@@ -617,8 +630,8 @@ static int net_layer_train_step(sb_net *net, int layer, const void *h_in, const 
   int rc = drop_frozen_cache(net);  // the layer changes: what was computed from it is stale
   if (rc) return rc;
   ScopedDeviceBuffer bX, bY;
-  SB_HIP(hipMalloc(&bX.p, (size_t)rows * L.N * sizeof(T)));
-  SB_HIP(hipMalloc(&bY.p, (size_t)rows * L.M * sizeof(T)));
+  SB_HIP(dev_malloc(&bX.p, (size_t)rows * L.N * sizeof(T)));
+  SB_HIP(dev_malloc(&bY.p, (size_t)rows * L.M * sizeof(T)));
   SB_HIP(hipMemcpy(bX.p, h_in, (size_t)rows * L.N * sizeof(T), hipMemcpyHostToDevice));
   SB_HIP(hipMemcpy(bY.p, h_out, (size_t)rows * L.M * sizeof(T), hipMemcpyHostToDevice));
   rc = layer_train_step<T>(L, (const T *)bX.p, (const T *)bY.p, rows, h);
@@ -737,12 +750,14 @@ int sb_sync(void) {
   return 0;
 }
 
+long sb_allocation_calls(void) { return g_allocation_calls; }
+
 void *sb_stream(void) { return g_ctx.ready ? (void *)g_ctx.stream : nullptr; }
 
 int sb_malloc(void **d_ptr, size_t bytes) {
   SB_READY();
   SB_REQUIRE(d_ptr, "null pointer");
-  SB_HIP(hipMalloc(d_ptr, bytes ? bytes : 1));
+  SB_HIP(dev_malloc(d_ptr, bytes ? bytes : 1));
   return 0;
 }
 int sb_free(void *d_ptr) {
@@ -909,9 +924,9 @@ int sb_net_create(sb_net **net, int dtype) {
   sb_net *n = new sb_net();
   n->dtype = dtype;
   n->esize = dtype == SB_F32 ? 4 : 8;
-  hipError_t e = hipMalloc((void **)&n->d_correct, sizeof(unsigned long long));
-  if (e == hipSuccess) e = hipMalloc((void **)&n->d_unmasked, sizeof(unsigned long long));
-  if (e == hipSuccess) e = hipEventCreateWithFlags(&n->perm_copied, hipEventDisableTiming);
+  hipError_t e = dev_malloc((void **)&n->d_correct, sizeof(unsigned long long));
+  if (e == hipSuccess) e = dev_malloc((void **)&n->d_unmasked, sizeof(unsigned long long));
+  if (e == hipSuccess) e = (g_allocation_calls++, hipEventCreateWithFlags(&n->perm_copied, hipEventDisableTiming));
   if (e != hipSuccess) {
     if (n->d_correct) (void)hipFree(n->d_correct);
     if (n->d_unmasked) (void)hipFree(n->d_unmasked);
@@ -1024,6 +1039,15 @@ int sb_net_randomize_layer(sb_net *net, int layer, uint64_t seed, double density
                               : net_randomize_layer<double>(net, layer, seed, density);
 }
 
+int sb_net_set_frozen_cache_limit(sb_net *net, size_t bytes) {
+  SB_READY();
+  SB_REQUIRE(net, "null pointer");
+  net->frozen_cache_limit = bytes;
+  if (net->Hc && 2 * (size_t)net->Ns * (size_t)net->layers[net->Hc_layer].M * net->esize > bytes)
+    return drop_frozen_cache(net);
+  return 0;
+}
+
 int sb_net_set_training_data(sb_net *net, const void *h_images, const void *h_labels, long n_samples,
                              long n_features, long n_classes) {
   SB_READY();
@@ -1033,14 +1057,15 @@ int sb_net_set_training_data(sb_net *net, const void *h_images, const void *h_la
   int rc = sb_net_training_done(net);
   if (rc) return rc;
   const size_t xb = (size_t)n_samples * n_features * net->esize;
-  SB_HIP(hipMalloc(&net->X, xb));
+  SB_HIP(dev_malloc(&net->X, xb));
   SB_HIP(hipMemcpy(net->X, h_images, xb, hipMemcpyHostToDevice));
   if (h_labels) {
     const size_t yb = (size_t)n_samples * n_classes * net->esize;
-    SB_HIP(hipMalloc(&net->Y, yb));
+    SB_HIP(dev_malloc(&net->Y, yb));
     SB_HIP(hipMemcpy(net->Y, h_labels, yb, hipMemcpyHostToDevice));
   }
-  SB_HIP(hipMalloc((void **)&net->d_perm, (size_t)n_samples * sizeof(int64_t)));
+  SB_HIP(dev_malloc((void **)&net->d_perm, (size_t)n_samples * sizeof(int64_t)));
+  g_allocation_calls++;
   SB_HIP(hipHostMalloc((void **)&net->h_perm, (size_t)n_samples * sizeof(int64_t), hipHostMallocDefault));
   SB_HIP(hipEventRecord(net->perm_copied, g_ctx.stream));
   net->Ns = n_samples;

@@ -173,6 +173,39 @@ def test_classifier_epochs_follow_changes_below_them_f64(hb):
     assert np.array_equal(g.predict(Xt, B), r.predict(Xt, B))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_classifier_epochs_without_the_activation_cache_are_bit_identical(hb, dtype):
+    """The cache of the frozen layers' activations is an optimisation with a fallback: when it is not
+    affordable (here: a limit of zero bytes, and a limit lowered while a cache is held) every step runs the
+    forward passes of the layers below instead.  Both ways give the same bits."""
+    rng = np.random.default_rng(78)
+    n_pix, H, Mc, n_out, Ns, B = 40, 4, 12, 5, 200, 16
+    X, Y = synthetic_images(rng, Ns, n_pix), one_hot_labels(rng, Ns, n_out)
+    states = []
+    for limit in (None, 0, "lowered"):
+        net = build_two_layer(hb, 2 * n_pix, H, Mc, n_out, dict(MNIST_HP, l1_density=0.4), dtype, seed=5)
+        if limit == 0:
+            net.net.set_frozen_cache_limit(0)
+        np.random.seed(11)
+        net.fit(X, Y, B, [(0, 1)])
+        if limit == "lowered":
+            # one epoch with the cache, then the limit drops below what it takes and the rest runs without
+            net.net.initiate_training(X.astype(dtype), Y.astype(dtype))
+            for epoch in range(3):
+                idx = np.random.permutation(Ns).astype(np.int64)
+                hc = np.random.permutation(1).astype(np.int64)
+                net.net.train_epoch(1, B, idx, hc, epoch)
+                if epoch == 0:
+                    net.net.set_frozen_cache_limit(1000)
+            net.net.training_done()
+        else:
+            net.fit(X, Y, B, [(1, 3)])
+        states.append({name: np.array(getattr(net._layers[1], name)) for name in ("Ci", "Cj", "Cij", "weights", "bias")})
+    for other in states[1:]:
+        for name, value in states[0].items():
+            assert np.array_equal(value, other[name]), name
+
+
 def test_small_network_one_epoch_f32(hb):
     # float32, one epoch per layer (13 batches, short last one).  Stated drift bound after one epoch:
     # 1e-5 relative (rounding differences of ~1e-7 per step, amplified by the log of small traces).
