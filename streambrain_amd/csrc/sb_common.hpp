@@ -123,6 +123,16 @@ __device__ __forceinline__ void load_vw(T (&out)[Real<T>::VW], const T *row, lon
   }
 }
 
+// A pointer whose value is the same in every lane, moved to scalar registers (the compiler does not always
+// see that it is, and a buffer descriptor built from vector registers costs a loop over the distinct values).
+template <typename T>
+__device__ __forceinline__ T *uniform_pointer(T *p) {
+  const unsigned long long b = reinterpret_cast<unsigned long long>(p);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b);
+  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+  return reinterpret_cast<T *>(((unsigned long long)hi << 32) | lo);
+}
+
 // A bounds-checked window of at most 2 GiB onto a global array, addressed through a buffer descriptor
 // with 32-bit byte offsets: a per-lane offset plus a wavefront-uniform one that lives in a scalar
 // register.  Accesses past the end of the window read zero and store nothing, in hardware; so a loop

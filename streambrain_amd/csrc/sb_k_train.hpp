@@ -19,7 +19,7 @@
 //      stored as 16-byte vectors straight from the accumulator registers (no pass through LDS).  The
 //      slabs are double-buffered and the global loads of two chunks are in flight: chunk c is staged from
 //      its registers, the registers take the loads of chunk c+2, and one barrier per chunk separates the
-//      staging from the MFMA loop.
+//      staging from the MFMA loop (at the start, chunk 1 is requested only once chunk 0 has been staged).
 //   2. From the same LDS slabs, the lanes of one wavefront add up one column each of x, those of
 //      another one column each of y (which two wavefronts rotates with the tile index), in batch order
 //      b = 0..B-1 without FMA contraction: the reference's summation order, so Ci, Cj and kbi stay
@@ -227,8 +227,12 @@ void k_train_fused(TrainArgs<T> a) {
     ynext += KC * M;
     rows_left -= rows;
   };
+  // Only chunk 0 is requested here; chunk 1 follows once chunk 0 sits in LDS (see `chunk`).  The five workgroups
+  // of a CU start together, and what they wait for first is chunk 0: with both chunks requested up front the
+  // CU's first-slab traffic doubles and the first MFMAs start later (1568 x 3000, batch 128: 0.25 us per launch;
+  // the mask bytes and old traces, which only the epilogue needs, likewise wait until the tile is requested:
+  // another 0.1 us).
   request_chunk(std::integral_constant<int, 0>{});
-  request_chunk(std::integral_constant<int, 1>{});
 
   // ---- this lane's share of the tile, in the layout the MFMA leaves it in: wavefront w owns tile rows
   // 16 w .. 16 w + 15 and all 64 columns as four 16 x 16 blocks; the B operand of block c is column
@@ -249,10 +253,10 @@ void k_train_fused(TrainArgs<T> a) {
   }
   const unsigned vstep = rstep * M * ES;  // from acc[..][v] to acc[..][v + 1] (uniform)
 
-  // mask bytes of the lane's synapses: a small, L2-resident array, fetched up front
+  // mask bytes of the lane's synapses: a small, L2-resident array, requested together with the Cij tile
   const bool masked = a.wmask != nullptr;
   uint32_t mb[4][NG][MB];
-  {
+  auto request_mask = [&]() {
     const ByteWindow mwin(masked ? a.wmask + (long)i0 * a.H : nullptr, tile_rows * a.H);
     const unsigned H = (unsigned)a.H;
 #pragma unroll
@@ -265,7 +269,7 @@ void k_train_fused(TrainArgs<T> a) {
         // scalar offset is added after that check)
         for (int v = 0; v < 4; v++) mb[v][g][e] = mwin.load((r0 + v * rstep) * H + hc, 0);
       }
-  }
+  };
 
   // column sums: one wavefront takes the 64 x columns of the tile (a lane each), one the 64 y columns,
   // the other two take none; which wavefronts do rotates with the tile, so that over the tiles of a
@@ -277,13 +281,18 @@ void k_train_fused(TrainArgs<T> a) {
   const bool sum_ok = summer && sidx < (sum_i ? N : M);
   const bool writes_bias = !PRE && sum_ok && !sum_i && it == 0 && a.bias_mode == 1;
   // old trace; with PRE the new one, which the same two wavefronts turn into the reciprocals below
-  const T cold = (PRE ? (sum_i ? a.Ci_next : a.Cj_next) : (sum_i ? a.Ci : a.Cj))[sum_ok ? sidx : 0];
-  T kb = T(1);
-  if (!PRE && a.bias_mode == 1) kb = a.kbi[writes_bias ? sidx : 0];
+  // (requested together with the Cij tile; unguarded, like every load here)
+  T cold = T(0), kb = T(1);
+  auto request_old_traces = [&]() {
+    cold = (PRE ? (sum_i ? a.Ci_next : a.Cj_next) : (sum_i ? a.Ci : a.Cj))[sum_ok ? sidx : 0];
+    if (!PRE && a.bias_mode == 1) kb = a.kbi[writes_bias ? sidx : 0];
+  };
   T csum = T(0);
 
   T cpre[4][NG][VW];  // Cij tile
   auto request_tile = [&]() {
+    request_mask();
+    request_old_traces();
 #pragma unroll
     for (int v = 0; v < 4; v++)
 #pragma unroll
@@ -292,8 +301,9 @@ void k_train_fused(TrainArgs<T> a) {
         // instruction's scalar offset is added after the range check, so with the step passed there a lane whose
         // first row is the tile's last would read rows past the tile (past the matrix, in the last tile row).
         const unsigned skip = v * vstep;
-        const BufferWindow<T> win(a.Cij + (long)i0 * a.M + (long)v * rstep * a.M,
-                                  typename BufferWindow<T>::Bytes{tile_bytes > skip ? tile_bytes - skip : 0u});
+        const unsigned left = __builtin_amdgcn_readfirstlane(tile_bytes > skip ? tile_bytes - skip : 0u);
+        const BufferWindow<T> win(uniform_pointer(a.Cij + (long)i0 * a.M + (long)v * rstep * a.M),
+                                  typename BufferWindow<T>::Bytes{left});
         win.load_vec(cpre[v][g], tat[g], 0);
       }
   };
@@ -336,7 +346,8 @@ void k_train_fused(TrainArgs<T> a) {
   // loads have two chunks' worth of MFMAs to arrive in.  One barrier per chunk: it publishes the slab, and
   // since every wavefront reaches it only after its MFMA loop over the previous chunk, the buffer written in
   // the next turn (read last two chunks ago) is free by then.
-  auto chunk = [&](auto set, auto with_tile, auto last) {
+  long t = 1;  // turn of two chunks
+  auto chunk = [&](auto set, auto with_tile, auto last, auto first) {
     constexpr int S = decltype(set)::value;
     T *xs = xs2[S], *ys = ys2[S];
 #pragma unroll
@@ -349,6 +360,16 @@ void k_train_fused(TrainArgs<T> a) {
       }
       *reinterpret_cast<vec_t *>(&xs[(er + RPP * m) * XP + VW * eg]) = vx;
       *reinterpret_cast<vec_t *>(&ys[(er + RPP * m) * TS + VW * eg]) = vy;
+    }
+    // The batch's first chunk is the one that requests chunk 1 (`first`: 0 never the first chunk, 1 always, 2
+    // in the first turn of the loop over turns).  The request has to stay behind the staging stores above:
+    // moved up by the compiler, ahead of the wait for chunk 0, it would be the early request again -- the
+    // uniform branch and the scheduling fence keep it in place.
+    if constexpr (decltype(first)::value == 2) {
+      if (t == 1) request_chunk(std::integral_constant<int, 1>{});
+    } else if constexpr (decltype(first)::value == 1) {
+      __builtin_amdgcn_sched_barrier(0);
+      request_chunk(std::integral_constant<int, 1>{});
     }
     request_chunk(set);  // chunk c + 2; past the batch: reads zeros nobody consumes
     if (decltype(with_tile)::value) request_tile();
@@ -430,27 +451,39 @@ void k_train_fused(TrainArgs<T> a) {
   constexpr std::false_type no{};
   constexpr std::true_type yes{};
   const long turns = (a.B + 2 * KC - 1) / (2 * KC);
-  long t = 1;
+  constexpr std::integral_constant<int, 0> f0{};
+  constexpr std::integral_constant<int, 1> f1{};
+  constexpr std::integral_constant<int, 2> f2{};
   if constexpr (sizeof(T) == 8) {
-    for (; t < turns; t++) {
-      chunk(set0, no, no);
-      chunk(set1, no, no);
-    }
-    chunk(set0, yes, no);
-    chunk(set1, no, yes);
-  } else {
-    for (; t + 1 < turns; t++) {
-      chunk(set0, no, no);
-      chunk(set1, no, no);
-    }
     if (turns >= 2) {
-      chunk(set0, no, no);
-      chunk(set1, yes, no);
-      chunk(set0, no, no);
-      chunk(set1, no, yes);
+      for (; t < turns; t++) {
+        chunk(set0, no, no, f2);
+        chunk(set1, no, no, f0);
+      }
+      chunk(set0, yes, no, f0);
+      chunk(set1, no, yes, f0);
     } else {
-      chunk(set0, yes, no);
-      chunk(set1, no, yes);
+      chunk(set0, yes, no, f1);
+      chunk(set1, no, yes, f0);
+    }
+  } else {
+    if (turns >= 3) {
+      for (; t + 1 < turns; t++) {
+        chunk(set0, no, no, f2);
+        chunk(set1, no, no, f0);
+      }
+      chunk(set0, no, no, f0);
+      chunk(set1, yes, no, f0);
+      chunk(set0, no, no, f0);
+      chunk(set1, no, yes, f0);
+    } else if (turns == 2) {
+      chunk(set0, no, no, f1);
+      chunk(set1, yes, no, f0);
+      chunk(set0, no, no, f0);
+      chunk(set1, no, yes, f0);
+    } else {
+      chunk(set0, yes, no, f1);
+      chunk(set1, no, yes, f0);
     }
   }
 
