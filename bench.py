@@ -6,6 +6,7 @@
   python bench.py --achievable-peaks                                   device-copy and matrix-core probes
   python bench.py --copy-calibration                                   known-size copies for counter scaling
   python bench.py --entry-point-rates                                  the per-function C entry points on their own
+  python bench.py --passes                                             trace, weight and forward passes one by one
   python bench.py --pmc-summary DIR                                    text summary of rocprofv3 --pmc runs
 
 Headline workload: the MNIST-shaped 2-layer network, float32, batch 128, 60000 seeded
@@ -401,6 +402,7 @@ def headline(args):
         "kernels": prof,
         "event_bracket_overhead_us": {"calibrated": bracket_us,
                                       "empty_bracket": run.lib.sb_profile_bracket_overhead_us()},
+        "passes": measure_passes(),
         "other_phases": {
             "classifier_layer_train_samples_per_s": cls_samples / cls_dt,
             "classifier_layer_train_first_epoch_samples_per_s": cls_samples / cls_first_dt,
@@ -753,6 +755,108 @@ def entry_point_rates(reps=200):
     return 0
 
 
+def measure_passes(reps=300):
+    """The passes of the training step one by one at the headline layer's shape (1568 -> 30 x 100, float32,
+    batch 128, mask density 0.1), each through its own C entry point on device buffers, `reps` launches back
+    to back, timed twice: wall clock per call without brackets, and with every launch bracketed by HIP
+    events on the library's stream (the headline's per-kernel brackets).  For the passes that are one launch
+    per call the first is the launch's duration, and their difference is what a bracket adds; the trace pass's
+    entry point is two launches (the training kernel, then the copy of the new Ci / Cj over the caller's), so
+    its kernel is priced from its brackets minus that difference:
+      trace pass     Ci/Cj/Cij moving averages, the Cij one as the MFMA GEMM x^T y with the decay in its
+                     epilogue (sb_update_counters: the fused training kernel without the weights)
+      weight pass    W = log(max(Cij, cthr^4) / (Ci Cj)) streamed over Cij (sb_weights_from_counters), and
+                     the same with the mask apply fused in (sb_weights_masked_from_counters)
+      forward        the dense x.W + bias GEMM with the softmax epilogue (sb_compute_activation)
+    Rates are on the algorithmic bytes / flops of each pass, against the published peaks."""
+    from streambrain_amd import _capi
+    from streambrain_amd._capi import DeviceArray
+    _capi.init(0)
+    lib, c = _capi.lib(), _capi.check
+    n, h, mc, b, es = 2 * N_PIXELS, H, MC, BATCH, 4
+    m = h * mc
+    rng = np.random.default_rng(0)
+    f = np.float32
+    x = DeviceArray.from_numpy((rng.random((b, n)) * (rng.random((b, n)) < 0.6)).astype(f))
+    act = DeviceArray.from_numpy(numpy_softmax(rng.standard_normal((b, m)), h, mc).astype(f))
+    out = DeviceArray((b, m), f)
+    W = DeviceArray.from_numpy((0.1 * rng.standard_normal((n, m))).astype(f))
+    bias = DeviceArray.from_numpy((0.1 * rng.random(m)).astype(f))
+    Ci = DeviceArray.from_numpy((0.3 + 0.1 * rng.random(n)).astype(f))
+    Cj = DeviceArray.from_numpy((0.005 + 0.01 * rng.random(m)).astype(f))
+    Cij = DeviceArray.from_numpy((0.003 * (0.1 + rng.random((n, m)))).astype(f))
+    mask_host = (rng.random((n, h)) < HP["l1_density"]).astype(np.uint8)
+    wmask = DeviceArray.from_numpy(mask_host)
+    connected = int(mask_host.sum()) * mc
+    tau, cthr = HP["l1_taupdt"], HP["l1_taupdt"] / 2
+    R = ctypes.c_float
+    calls = {
+        "trace": (lambda: lib.sb_update_counters_f32(Ci.ptr, Cj.ptr, Cij.ptr, x.ptr, act.ptr, R(tau), b, n, m),
+                  "train_fused"),
+        "weight": (lambda: lib.sb_weights_from_counters_f32(W.ptr, Ci.ptr, Cj.ptr, Cij.ptr, R(cthr), n, m),
+                   "weight_pass"),
+        "weight_masked": (lambda: lib.sb_weights_masked_from_counters_f32(W.ptr, Ci.ptr, Cj.ptr, Cij.ptr, wmask.ptr,
+                                                                          R(cthr), n, h, mc), "weight_pass"),
+        "forward_dense": (lambda: lib.sb_compute_activation_f32(out.ptr, x.ptr, W.ptr, bias.ptr, b, n, h, mc),
+                          "forward"),
+    }
+    measured = {}
+    for name, (call, kernel) in calls.items():
+        for _ in range(20):
+            c(call())
+        c(lib.sb_sync())
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            c(call())
+        c(lib.sb_sync())
+        wall_us = 1e6 * (time.perf_counter() - t0) / reps
+        c(lib.sb_profile_start())
+        for _ in range(reps):
+            c(call())
+        c(lib.sb_profile_stop())
+        prof, _, _ = read_profile(lib, c)
+        measured[name] = {"launches": prof[kernel]["launches"], "raw_avg_us": prof[kernel]["raw_avg_us"],
+                          "wall_us_per_call_back_to_back": wall_us}
+    singles = sorted(measured[k]["raw_avg_us"] - measured[k]["wall_us_per_call_back_to_back"]
+                     for k in ("weight", "weight_masked", "forward_dense"))
+    bracket_us = max(singles[1], 0.0)
+    for name, v in measured.items():
+        v["avg_us"] = v["raw_avg_us"] - bracket_us if name == "trace" else v["wall_us_per_call_back_to_back"]
+    gemm = 2.0 * b * n * m
+    peak = MFMA_PEAK_TFLOPS["f32"]
+
+    def hbm(t_us, nbytes):
+        return {"algorithmic_bytes": nbytes, "GBps": nbytes / (t_us * 1e-6) / 1e9,
+                "frac_of_hbm_peak": nbytes / (t_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+
+    def mfma(t_us, flops):
+        return {"flops": flops, "TFLOPps": flops / (t_us * 1e-6) / 1e12,
+                "frac_of_mfma_peak": flops / (t_us * 1e-6) / 1e12 / peak}
+
+    t = {k: v["avg_us"] for k, v in measured.items()}
+    passes = {
+        "shape": {"in_features": n, "hypercolumns": h, "minicolumns": mc, "batch": b, "mask_density": HP["l1_density"],
+                  "dtype": "f32"},
+        "how": f"{reps} calls back to back per pass; avg_us = wall clock per call for the one-launch passes, "
+               "bracketed average minus what a bracket adds for the trace pass",
+        "event_bracket_overhead_us": bracket_us,
+        "trace": dict(measured["trace"], kernel="k_train_fused, traces only (sb_update_counters; the Ci / Cj copy "
+                                                "back of that entry point is a separate launch, not timed here)",
+                      mfma=mfma(t["trace"], gemm), hbm=hbm(t["trace"], 2 * es * n * m + es * b * (n + m))),
+        "weight": dict(measured["weight"], kernel="k_weight_pass, no mask (sb_weights_from_counters)",
+                       hbm=hbm(t["weight"], 2 * es * n * m)),
+        "weight_masked": dict(measured["weight_masked"],
+                              kernel="k_weight_pass with the mask apply (sb_weights_masked_from_counters)",
+                              hbm=hbm(t["weight_masked"], 2 * es * n * m + n * h),
+                              bytes_the_kernel_must_move_at_this_mask_density=es * n * m + es * connected + n * h),
+        "forward_dense": dict(measured["forward_dense"], kernel="k_forward (sb_compute_activation, dense W)",
+                              mfma=mfma(t["forward_dense"], gemm)),
+    }
+    for d in (x, act, out, W, bias, Ci, Cj, Cij, wmask):
+        d.free()
+    return passes
+
+
 def _pmc_medians(directory):
     import collections
     import csv
@@ -823,6 +927,9 @@ def main():
                          "next to the published peaks)")
     ap.add_argument("--entry-point-rates", action="store_true",
                     help="only time the per-function entry points of the C ABI at the headline layer's shape")
+    ap.add_argument("--passes", action="store_true",
+                    help="only time the passes of the training step one by one (trace, weight, forward) at the "
+                         "headline layer's shape")
     ap.add_argument("--pmc-summary", metavar="DIR", help="summarise rocprofv3 --pmc csv output below DIR")
     ap.add_argument("--pmc-calibration", metavar="DIR",
                     help="with --pmc-summary: the same counters over `bench.py --copy-calibration`")
@@ -839,6 +946,9 @@ def main():
         return achievable_peaks()
     if args.entry_point_rates:
         return entry_point_rates()
+    if args.passes:
+        print(json.dumps({"passes": measure_passes()}))
+        return 0
     if args.workload != "mnist":
         cfg = LARGE[args.workload]
         nb = (cfg["samples"] + cfg["batch"] - 1) // cfg["batch"]

@@ -118,6 +118,13 @@ int sb_weights_from_counters_f32(float *d_W, const float *d_Ci, const float *d_C
                                  float cthr, long N, long M);
 int sb_weights_from_counters_f64(double *d_W, const double *d_Ci, const double *d_Cj, const double *d_Cij,
                                  double cthr, long N, long M);
+/* sb_weights_from_counters followed by sb_apply_mask in one pass over Cij and W (the weight recompute fused
+ * with the mask apply: kernels_openmp_internal.cc:192-199 then :322-335): W[i, j] is the weight where
+ * wmask[i, j / Mc] is set and 0 elsewhere; Cij under zero mask bytes is not read. */
+int sb_weights_masked_from_counters_f32(float *d_W, const float *d_Ci, const float *d_Cj, const float *d_Cij,
+                                        const uint8_t *d_wmask, float cthr, long N, long H, long Mc);
+int sb_weights_masked_from_counters_f64(double *d_W, const double *d_Ci, const double *d_Cj, const double *d_Cij,
+                                        const uint8_t *d_wmask, double cthr, long N, long H, long Mc);
 int sb_add_bias_f32(float *d_act, const float *d_bias, long B, long M);
 int sb_add_bias_f64(double *d_act, const double *d_bias, long B, long M);
 

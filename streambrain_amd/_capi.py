@@ -27,6 +27,7 @@ _KERNEL_SIGS = {
     "sb_update_weights": lambda R: [_P, _P, _P, _P, _P, R, _P, R, _L, _L, _L],
     "sb_update_counters": lambda R: [_P, _P, _P, _P, _P, R, _L, _L, _L],
     "sb_weights_from_counters": lambda R: [_P, _P, _P, _P, R, _L, _L],
+    "sb_weights_masked_from_counters": lambda R: [_P, _P, _P, _P, _P, R, _L, _L, _L],
     "sb_add_bias": lambda R: [_P, _P, _L, _L],
     "sb_update_bias": lambda R: [_P, _P, R, _L],
     "sb_update_bias_regularized": lambda R: [_P, _P, _P, R, R, R, R, _L],

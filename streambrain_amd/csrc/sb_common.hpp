@@ -257,6 +257,19 @@ struct BufferWindow {
   }
 };
 
+// A raw byte window (for mask bytes): bounds-checked like BufferWindow.
+struct ByteWindow {
+  __amdgpu_buffer_rsrc_t rsrc;
+  __device__ ByteWindow(const uint8_t *base, long bytes) {
+    const long b = (base && bytes > 0) ? bytes : 0;
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0,
+                                             (int)(unsigned)(b < 0x80000000L ? b : 0x80000000L), 0x00020000);
+  }
+  __device__ __forceinline__ uint32_t load(unsigned at, unsigned uniform) const {
+    return __builtin_amdgcn_raw_buffer_load_b8(rsrc, (int)at, (int)uniform, 0);
+  }
+};
+
 // Exchange inside a row of 16 lanes with data-parallel-primitive moves (no LDS round trip).  The four
 // controls below -- swap neighbours, swap pairs, mirror each half row, mirror the row -- applied in
 // turn with a commutative pick leave the row-wide result in every one of the 16 lanes.

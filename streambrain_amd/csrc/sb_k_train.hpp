@@ -123,19 +123,6 @@ __global__ __launch_bounds__(256) void k_trace_sums(TrainArgs<T> a) {
 template <typename T, bool VEC, int MB>
 constexpr int train_waves_per_simd() { return sizeof(T) == 8 ? 4 : (VEC && MB == 1 ? 5 : 4); }
 
-// A raw byte window (for the mask bytes of a tile's rows): bounds-checked like BufferWindow.
-struct ByteWindow {
-  __amdgpu_buffer_rsrc_t rsrc;
-  __device__ ByteWindow(const uint8_t *base, long bytes) {
-    const long b = (base && bytes > 0) ? bytes : 0;
-    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0,
-                                             (int)(unsigned)(b < 0x80000000L ? b : 0x80000000L), 0x00020000);
-  }
-  __device__ __forceinline__ uint32_t load(unsigned at, unsigned uniform) const {
-    return __builtin_amdgcn_raw_buffer_load_b8(rsrc, (int)at, (int)uniform, 0);
-  }
-};
-
 // VEC: Cij and W are stored as 16-byte vectors (M a multiple of VW), element by element otherwise.  Loads
 // are 16-byte accesses either way: one that runs over the end of a row of x, y or Cij fetches elements of
 // the next row into tile rows / columns outside the matrix, which are never stored or summed.

@@ -86,38 +86,64 @@ __global__ __launch_bounds__(256) void k_weights_from_traces(T *W, const T *Ci, 
   }
 }
 
-// The same for M a multiple of VW and 16-byte aligned arrays: a thread owns VW consecutive columns (their
-// column reciprocals computed once) and walks kRowsPerTurn rows per turn with 16-byte accesses, all loads
-// of a turn in flight before the first is used.  Grid: x over blocks of 256 VW columns, y over row groups.
+// The weight pass on its own, with or without the mask (omp.cc:192-199 followed by apply_mask, :322-335):
+//   W[i, j] = wmask[i, j / Mc] ? log(max(Cij, cthr^4) / (Ci Cj)) : 0      (0 as well where Ci or Cj < cthr)
+// for rows that are whole 16-byte vectors (M, and with a mask Mc, multiples of VW).  Bound by HBM: it reads Cij
+// and writes W once, 2 s N M bytes, plus the N H mask bytes.  A thread owns VW consecutive columns (their
+// column reciprocals computed once) of kRowsPerTurn rows: all its loads are in flight before the first is used.
+// Cij and W are reached through bounds-checked windows over the rows of a turn (rows past the matrix read
+// zero and store nothing), so the loop has no guards; under a zero mask byte the Cij vector is not read at all
+// (an offset outside the window costs no memory access), and with `w_masked` -- the caller vouches that W
+// holds zero there already -- not written either.  Stores write through (agent scope): with the default
+// policy they sit in the L2s until the kernel ends and are written back then, which is serial time.
+// Grid: x over blocks of 256 VW columns, y over row groups.
 constexpr int kRowsPerTurn = 8;
-template <typename T>
-__global__ __launch_bounds__(256) void k_weights_from_traces_vec(T *W, const T *Ci, const T *Cj, const T *Cij,
-                                                                 T cthr, T cthr4, long N, long M) {
+template <typename T, bool MASKED>
+__global__ __launch_bounds__(256) void k_weight_pass(T *W, const T *Ci, const T *Cj, const T *Cij,
+                                                     const uint8_t *wmask, T cthr, T cthr4, long N, long M, long H,
+                                                     FastDiv by_Mc, int w_masked) {
   constexpr int VW = Real<T>::VW;
+  constexpr unsigned ES = sizeof(T), kOutside = BufferWindow<T>::kOutside;
   using vec_t = typename Real<T>::vec_t;
   const long j = ((long)blockIdx.x * 256 + threadIdx.x) * VW;
-  if (j >= M) return;
-  const vec_t cj = *reinterpret_cast<const vec_t *>(Cj + j);
+  const bool col_ok = j < M;
   T rcj[VW];
+  {
+    const BufferWindow<T> jwin(Cj, M);
+    T cj[VW];
+    jwin.load_vec(cj, col_ok ? (unsigned)j * ES : kOutside, 0);
 #pragma unroll
-  for (int e = 0; e < VW; e++) rcj[e] = trace_reciprocal<T>(cj[e], cthr);
+    for (int e = 0; e < VW; e++) rcj[e] = trace_reciprocal<T>(cj[e], cthr);
+  }
+  const unsigned hc = MASKED && col_ok ? by_Mc.div((uint32_t)j) : 0u;
+  const unsigned row_bytes = (unsigned)M * ES;  // kRowsPerTurn rows stay below 2 GiB (launcher)
   for (long i0 = (long)blockIdx.y * kRowsPerTurn; i0 < N; i0 += (long)gridDim.y * kRowsPerTurn) {
-    vec_t c[kRowsPerTurn];
-    T rci[kRowsPerTurn];
+    const long rows = N - i0 < kRowsPerTurn ? N - i0 : kRowsPerTurn;
+    const unsigned turn_bytes = (unsigned)rows * row_bytes;
+    const BufferWindow<T> cwin(uniform_pointer(Cij + i0 * M), typename BufferWindow<T>::Bytes{turn_bytes}),
+        wwin(uniform_pointer(W + i0 * M), typename BufferWindow<T>::Bytes{turn_bytes});
+    uint32_t on[kRowsPerTurn];
+    if constexpr (MASKED) {
+      const ByteWindow mwin(uniform_pointer(wmask + i0 * H), rows * H);
+#pragma unroll
+      for (int r = 0; r < kRowsPerTurn; r++) on[r] = mwin.load((unsigned)(r * H) + hc, 0);
+    }
+    T c[kRowsPerTurn][VW], ci[kRowsPerTurn];
 #pragma unroll
     for (int r = 0; r < kRowsPerTurn; r++) {
-      const long i = i0 + r < N ? i0 + r : N - 1;
-      c[r] = *reinterpret_cast<const vec_t *>(Cij + i * M + j);
-      rci[r] = Ci[i];
+      const bool connected = !MASKED || on[r] != 0;
+      cwin.load_vec(c[r], col_ok && connected ? r * row_bytes + (unsigned)j * ES : kOutside, 0);
+      ci[r] = Ci[i0 + r < N ? i0 + r : N - 1];
     }
 #pragma unroll
     for (int r = 0; r < kRowsPerTurn; r++) {
-      if (i0 + r >= N) break;
-      const T ri = trace_reciprocal<T>(rci[r], cthr);
-      vec_t w;
+      const bool connected = !MASKED || on[r] != 0;
+      const T ri = trace_reciprocal<T>(ci[r], cthr);
+      T w[VW];
 #pragma unroll
-      for (int e = 0; e < VW; e++) w[e] = weight_from_traces<T>(c[r][e], ri, rcj[e], cthr4);
-      *reinterpret_cast<vec_t *>(W + (i0 + r) * M + j) = w;
+      for (int e = 0; e < VW; e++) w[e] = connected ? weight_from_traces<T>(c[r][e], ri, rcj[e], cthr4) : T(0);
+      const bool skip = MASKED && w_masked && !connected;
+      wwin.store_vec(w, col_ok && !skip ? r * row_bytes + (unsigned)j * ES : kOutside, 0);
     }
   }
 }
@@ -136,7 +162,7 @@ __global__ __launch_bounds__(256) void k_apply_mask(T *W, const uint8_t *wmask, 
 }
 
 // The same for M and Mc multiples of VW and a 16-byte aligned W: a thread owns VW consecutive columns (one
-// hypercolumn) and stores 16-byte zero vectors; nothing of W is read.  Grid as k_weights_from_traces_vec.
+// hypercolumn) and stores 16-byte zero vectors; nothing of W is read.  Grid as k_weight_pass.
 template <typename T>
 __global__ __launch_bounds__(256) void k_apply_mask_vec(T *W, const uint8_t *wmask, long N, long M, long H,
                                                         FastDiv by_Mc) {

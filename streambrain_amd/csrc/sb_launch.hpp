@@ -31,7 +31,7 @@ struct TraceScalars {
 // with a pair of HIP events on the launch stream; sb_profile_stop sums the elapsed times per kernel.
 enum KernelId {
   K_FORWARD = 0, K_SOFTMAX, K_UPDATE_BIAS, K_UPDATE_BIAS_REG, K_MASK_SCORES,
-  K_MASK_SWAP, K_MASK_FIX, K_APPLY_MASK, K_ARGMAX, K_GATHER, K_FILL, K_TRAIN_FUSED, K_MASK_ROWS, K_COUNT
+  K_MASK_SWAP, K_MASK_FIX, K_APPLY_MASK, K_ARGMAX, K_GATHER, K_FILL, K_TRAIN_FUSED, K_MASK_ROWS, K_WEIGHT_PASS, K_COUNT
 };
 const char *kernel_name(int id);
 struct ProfScope {
@@ -91,10 +91,11 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
                        T *Ci_next, T *Cj_next, const uint8_t *wmask, int bias_mode, T *bias, T *kbi,
                        long B, long N, long H, long Mc, T taupdt, T cthr, T khalf, T pmin, T taubdt,
                        bool w_masked);
-// W from the traces as they are, the fused kernel's expression (unmasked).
+// W from the traces as they are, the fused kernel's expression; wmask != nullptr: zero under zero mask bytes
+// (w_masked: the caller vouches that W is zero there already, and such entries are left alone).
 template <typename T>
-int launch_weights_from_traces(hipStream_t st, T *W, const T *Ci, const T *Cj, const T *Cij, T cthr, long N,
-                               long M);
+int launch_weights_from_traces(hipStream_t st, T *W, const T *Ci, const T *Cj, const T *Cij, const uint8_t *wmask,
+                               T cthr, long N, long H, long Mc, bool w_masked);
 template <typename T>
 int launch_add_bias(hipStream_t st, T *act, const T *bias, long B, long M);
 template <typename T>

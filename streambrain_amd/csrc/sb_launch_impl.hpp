@@ -319,23 +319,32 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
 }
 
 template <typename T>
-int launch_weights_from_traces(hipStream_t st, T *W, const T *Ci, const T *Cj, const T *Cij, T cthr, long N,
-                               long M) {
+int launch_weights_from_traces(hipStream_t st, T *W, const T *Ci, const T *Cj, const T *Cij, const uint8_t *wmask,
+                               T cthr, long N, long H, long Mc, bool w_masked) {
   SB_REQUIRE(W && Ci && Cj && Cij, "null pointer");
-  SB_REQUIRE(N > 0 && M > 0, "sizes must be positive");
+  SB_REQUIRE(N > 0 && H > 0 && Mc > 0, "sizes must be positive");
+  const long M = H * Mc;
+  SB_REQUIRE(M < (1L << 31) && N < (1L << 31), "dimension too large");
   const TraceScalars<T> s = TraceScalars<T>::from(T(0), cthr);
-  ProfScope prof_(st, K_APPLY_MASK);
+  ProfScope prof_(st, K_WEIGHT_PASS);
   constexpr int VW = Real<T>::VW;
-  if (M % VW == 0 && aligned16(W) && aligned16(Cij) && aligned16(Cj)) {
+  // 16-byte vectors that lie inside one row (and one hypercolumn), and a turn's rows inside one window
+  if (M % VW == 0 && (!wmask || Mc % VW == 0) && kRowsPerTurn * M * (long)sizeof(T) < (1L << 31)) {
     const long turns = cdiv(N, kRowsPerTurn);
-    hipLaunchKernelGGL((k_weights_from_traces_vec<T>), dim3((unsigned)cdiv(M, 256 * VW), (unsigned)(turns < 4096 ? turns : 4096)),
-                       dim3(256), 0, st, W, Ci, Cj, Cij, cthr, s.cthr4, N, M);
+    const dim3 grid((unsigned)cdiv(M, 256 * VW), (unsigned)(turns < 32768 ? turns : 32768));
+    if (wmask)
+      hipLaunchKernelGGL((k_weight_pass<T, true>), grid, dim3(256), 0, st, W, Ci, Cj, Cij, wmask, cthr, s.cthr4, N, M,
+                         H, FastDiv::of(Mc), w_masked ? 1 : 0);
+    else
+      hipLaunchKernelGGL((k_weight_pass<T, false>), grid, dim3(256), 0, st, W, Ci, Cj, Cij, wmask, cthr, s.cthr4, N, M,
+                         H, FastDiv::of(Mc), 0);
     SB_LAUNCH_CHECK();
     return 0;
   }
   hipLaunchKernelGGL((k_weights_from_traces<T>), dim3((unsigned)(N < 8192 ? N : 8192)), dim3(256), 0, st, W, Ci,
                      Cj, Cij, cthr, s.cthr4, N, M);
   SB_LAUNCH_CHECK();
+  if (wmask) return launch_apply_mask<T>(st, W, wmask, N, H, Mc);
   return 0;
 }
 
@@ -581,8 +590,8 @@ int launch_copy_pair(hipStream_t st, T *dst1, const T *src1, size_t n1, T *dst2,
                                      T *, T *, const uint8_t *, int, T *, T *, long, long, long, long, \
                                      T, T, T, T, T, bool);                                             \
   template int launch_update_bias<T>(hipStream_t, T *, const T *, T, long);                           \
-  template int launch_weights_from_traces<T>(hipStream_t, T *, const T *, const T *, const T *, T,    \
-                                             long, long);                                             \
+  template int launch_weights_from_traces<T>(hipStream_t, T *, const T *, const T *, const T *,       \
+                                             const uint8_t *, T, long, long, long, bool);             \
   template int launch_add_bias<T>(hipStream_t, T *, const T *, long, long);                           \
   template int launch_update_bias_regularized<T>(hipStream_t, T *, T *, const T *, T, T, T, T, long); \
   template int launch_update_mask<T>(hipStream_t, uint8_t *, const T *, const T *, const T *,         \

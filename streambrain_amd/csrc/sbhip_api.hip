@@ -76,7 +76,7 @@ const char *kernel_name(int id) {
   static const char *names[K_COUNT] = {"forward", "softmax", "update_bias",
                                        "update_bias_regularized", "mask_scores", "mask_swap",
                                        "mask_fix_weights", "apply_mask", "argmax", "gather_rows", "fill",
-                                       "train_fused", "mask_rows"};
+                                       "train_fused", "mask_rows", "weight_pass"};
   return (id >= 0 && id < K_COUNT) ? names[id] : "?";
 }
 
@@ -841,7 +841,13 @@ int sb_fill_bytes(void *d_dst, int value, size_t bytes) {
   int sb_weights_from_counters_##SFX(T *W, const T *Ci, const T *Cj, const T *Cij, T cthr, long N,     \
                                      long M) {                                                         \
     SB_READY();                                                                                        \
-    return launch_weights_from_traces<T>(g_ctx.stream, W, Ci, Cj, Cij, cthr, N, M);                    \
+    return launch_weights_from_traces<T>(g_ctx.stream, W, Ci, Cj, Cij, nullptr, cthr, N, 1, M, false); \
+  }                                                                                                    \
+  int sb_weights_masked_from_counters_##SFX(T *W, const T *Ci, const T *Cj, const T *Cij,              \
+                                            const uint8_t *wmask, T cthr, long N, long H, long Mc) {   \
+    SB_READY();                                                                                        \
+    SB_REQUIRE(wmask, "null pointer");                                                                 \
+    return launch_weights_from_traces<T>(g_ctx.stream, W, Ci, Cj, Cij, wmask, cthr, N, H, Mc, false);  \
   }                                                                                                    \
   int sb_add_bias_##SFX(T *act, const T *bias, long B, long M) {                                       \
     SB_READY();                                                                                        \

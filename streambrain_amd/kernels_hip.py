@@ -153,6 +153,21 @@ def update_weights(*args):
     return _back(Ci, d_ci), _back(Cj, d_cj), _back(Cij, d_cij), _back(weights, d_w)
 
 
+def update_weights_masked(weights, Ci, Cj, Cij, cthr, wmask, hypercolumns, minicolumns):
+    """The weights from the traces as they are, zero under zero mask bytes: update_weights(weights, Ci, Cj,
+    Cij, cthr) followed by apply_mask(weights, wmask, hypercolumns, minicolumns) in one pass; returns weights."""
+    dt = weights.dtype
+    N, M = weights.shape
+    assert M == hypercolumns * minicolumns and Ci.shape == (N,) and Cj.shape == (M,) and Cij.shape == (N, M)
+    d_w = DeviceArray((N, M), dt)
+    d_ci, d_cj, d_cij = _dev(Ci, dt), _dev(Cj, dt), _dev(Cij, dt)
+    d_m = _dev(np.asarray(wmask).astype(np.uint8))
+    assert d_m.shape == (N, hypercolumns)
+    check(_fn("sb_weights_masked_from_counters", dt)(d_w.ptr, d_ci.ptr, d_cj.ptr, d_cij.ptr, d_m.ptr, cthr, N,
+                                                     hypercolumns, minicolumns))
+    return _back(weights, d_w)
+
+
 def update_bias(bias, Cj, cthr):
     dt = bias.dtype
     f = _fn("sb_update_bias", dt)

@@ -234,6 +234,28 @@ def test_update_counters_then_weights(k, oracle, dtype, B, N, M):
 
 
 @pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("N,H,Mc,density", [(5, 3, 4, 0.5), (37, 5, 12, 0.3), (130, 1, 64, 0.5), (257, 2, 65, 0.4),
+                                            (203, 7, 6, 0.0), (203, 7, 6, 1.0), (1568, 30, 100, 0.1)])
+def test_weights_masked_from_counters(k, oracle, dtype, N, H, Mc, density):
+    """The weight pass with the mask apply fused in (kernels_openmp_internal.cc:192-199 then :322-335 of the
+    reference) against the CPU restatement's two calls, and bit for bit against the GPU's own two calls."""
+    rng = np.random.default_rng(N + 31 * H + Mc)
+    M = H * Mc
+    x, y, Ci, Cj, Cij = _trace_problem(rng, 4, N, M, dtype)
+    cthr = 0.005
+    wmask = (rng.random((N, H)) < density).astype(np.uint8)
+    # taupdt = 0 leaves the traces as they are: the restatement's update_weights then is the weight pass alone
+    ref = oracle.update_weights(Ci.copy(), Cj.copy(), Cij.copy(), x, y, 0.0, np.zeros((N, M), dtype=dtype), cthr)
+    assert np.array_equal(ref[0], Ci) and np.array_equal(ref[2], Cij)
+    ref_w = oracle.apply_mask(ref[3].copy(), wmask, H, Mc)
+    got = k.update_weights_masked(np.full((N, M), 5.0, dtype=dtype), Ci, Cj, Cij, cthr, wmask, H, Mc)
+    assert_close(got, ref_w, dtype, "masked W")
+    assert np.array_equal(got == 0, ref_w == 0)
+    two = k.apply_mask(k.update_weights(np.full((N, M), 5.0, dtype=dtype), Ci, Cj, Cij, cthr), wmask, H, Mc)
+    assert np.array_equal(got, two)
+
+
+@pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("B,M", [(1, 1), (7, 33), (128, 3000)])
 def test_add_bias(k, dtype, B, M):
     rng = np.random.default_rng(B + M)
