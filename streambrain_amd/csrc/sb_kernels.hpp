@@ -231,35 +231,67 @@ struct MaskArgs {
 };
 constexpr int kMaxChangedRows = 64;  // rows that change sides in one merged launch: two per iteration
 
+// One wavefront per input row.  The score nominator is the reference's own expression, operation by operation
+// (omp.cc:257-277): every product, difference, quotient and sum rounded once, the logarithms accurate to the
+// last bit or so (evaluated in double and narrowed for floats), and the Mc terms of a row added in ascending
+// column order starting from zero -- so that two builds that start from the same traces pick the same rows.
+// The lanes evaluate 64 terms at a time; the sum then walks them in order (lane by lane through scalar
+// registers), which every lane does for itself.  Without a W array (the network path, where W is kept masked)
+// the weight is recomputed as the reference's weight pass forms it (omp.cc:192-199): log(max(Cij, cthr^4) /
+// (Ci Cj)) with the product and the quotient rounded like there.
+template <typename T>
+__device__ __forceinline__ T accurate_log(T x) {
+  if constexpr (sizeof(T) == 4) return (T)log((double)x);
+  else return log(x);
+}
 template <typename T>
 __global__ __launch_bounds__(256) void k_mask_scores(MaskArgs<T> a) {
+  using R = Real<T>;
   const int lane = threadIdx.x & 63;
   const long i = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (i >= a.N) return;
   const T pi = a.Ci[i];
-  const T rci = trace_reciprocal<T>(pi, a.cthr);
   T score = T(0);
-  if (pi >= a.cthr) {
-    for (long c = lane; c < a.Mc; c += 64) {
-      const long j = a.h * a.Mc + c;
+  if (pi >= a.cthr) {  // (uniform per wavefront)
+    const T omp = R::add(T(1), -pi);
+    for (long c0 = 0; c0 < a.Mc; c0 += 64) {
+      const long c = c0 + lane;
+      const long j = a.h * a.Mc + (c < a.Mc ? c : a.Mc - 1);
       const T pj = a.Cj[j];
-      if (pj >= a.cthr) {
+      T term = T(0);
+      if (c < a.Mc && pj >= a.cthr) {
         const T pij = a.Cij[i * a.M + j];
-        const T wij = a.W ? a.W[i * a.M + j]
-                          : weight_from_traces<T>(pij, rci, trace_reciprocal<T>(pj, a.cthr), a.cthr4);
-        const T xx = (T(1) - pi) * pj;
-        const T yy = (pj - pij) / xx;
-        score += pij * wij + (pj - pij) * Real<T>::log_(yy);
+        T wij;
+        if (a.W) {
+          wij = a.W[i * a.M + j];
+        } else {
+          const T num = pij > a.cthr4 ? pij : a.cthr4;  // cthr^4 as well when pij is NaN
+          wij = accurate_log<T>(R::div(num, R::mul(pi, pj)));
+        }
+        const T d = R::add(pj, -pij);
+        const T yy = R::div(d, R::mul(omp, pj));
+        term = R::add(R::mul(pij, wij), R::mul(d, accurate_log<T>(yy)));
+      }
+      // columns past the hypercolumn and columns below the threshold contribute an exact zero
+#pragma unroll
+      for (int k = 0; k < 64; k++) {
+        T tk;
+        if constexpr (sizeof(T) == 4) {
+          tk = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(term), k));
+        } else {
+          const long long b = __double_as_longlong(term);
+          const int lo = __builtin_amdgcn_readlane((int)(b & 0xffffffffLL), k);
+          const int hi = __builtin_amdgcn_readlane((int)(b >> 32), k);
+          tk = __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+        }
+        score = R::add(score, tk);
       }
     }
   }
   int cs = 0;
   for (long g = lane; g < a.H; g += 64) cs += a.wmask[i * a.H + g];
 #pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) {
-    score += __shfl_xor(score, o);
-    cs += __shfl_xor(cs, o);
-  }
+  for (int o = 32; o >= 1; o >>= 1) cs += __shfl_xor(cs, o);
   if (lane == 0) {
     a.nom[i] = score;
     a.csum[i] = cs;

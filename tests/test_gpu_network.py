@@ -313,10 +313,13 @@ def test_mnist_shape_rewiring_steps_f32(hb):
     is handed, with the state it started from, to the GPU's fused training step (traces, weights recomputed
     on the device, scores, swaps), and the two masks are compared.  Where they differ, the rows one side
     connected and the other did not (and likewise the rows disconnected) are paired in score order, and
-    every pair must be a near-tie: scores within 32 float32 rounding steps of each other (the scores are
-    sums of a hundred rounded terms built on logarithms the two sides evaluate with different routines).
-    The number of forked steps and the widest such pair are printed and recorded (measured: 19 of 30 steps
-    fork, 34 of 960 row decisions go to another row, the widest pair 17.9 rounding steps apart)."""
+    every pair must be a near-tie: scores within 4 float32 rounding steps of each other.  The device scores a
+    row the way the reference does, operation by operation and term by term in column order, so what is left
+    to differ between the two sides is the summation order of the batch inside Cij (matrix instructions
+    against a sequential loop).  The number of forked steps and the widest such pair are printed and recorded
+    (measured: 2 of 30 steps fork, 2 of 480 swaps go to another row, both exact ties of the float64 scores;
+    with the weights recomputed through the hardware logarithm and the terms added by a lane butterfly it
+    was 19 steps, 34 swaps and up to 17.9 rounding steps)."""
     from oracle import cpu_backend as ob
     from streambrain_amd import kernels_hip as k
     steps = []
@@ -370,13 +373,13 @@ def test_mnist_shape_rewiring_steps_f32(hb):
             for a, b in zip(mine, theirs):
                 gap = abs(score[a] - score[b]) / max(unit[a], unit[b])
                 widest = max(widest, gap)
-                assert gap <= 32, (f"hypercolumn {h}: rows {a} and {b} were decided differently although their "
+                assert gap <= 4, (f"hypercolumn {h}: rows {a} and {b} were decided differently although their "
                                    f"scores are {gap:.1f} rounding steps apart")
     print(f"rewiring steps: {30 - forks} equal, {forks} forked; {differing} of {swaps_total} swaps went to another "
           f"row, the widest such pair {widest:.1f} float32 rounding steps apart")
     record_error("forked rewiring steps of 30", forks, 30)
     record_error("swaps that went to another row", differing, swaps_total)
-    record_error("widest forked pair (rounding steps)", widest, 32)
+    record_error("widest forked pair (rounding steps)", widest, 4)
     assert swaps_total > 250, "the run is meant to rewire"
 
 
