@@ -30,9 +30,14 @@ import hashlib
 import json
 import os
 import sys
+import tempfile
 import time
 
-import numpy as np
+# thread placement of the CPU baseline's OpenMP loops (read when the OpenMP runtime first starts)
+os.environ.setdefault("OMP_PROC_BIND", "close")
+os.environ.setdefault("OMP_PLACES", "cores")
+
+import numpy as np  # noqa: E402
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
@@ -146,8 +151,12 @@ def cpu_baseline(x, st, h, mc, batch, tau, dtype, budget_s, min_steps=1, rewire_
     `rewire_period`-th step; at least min_steps timed steps, then until budget_s is used up."""
     from concurrent.futures import ThreadPoolExecutor
     from threadpoolctl import threadpool_limits
+    from oracle import build as oracle_build
     from oracle.oracle import Oracle
-    o = Oracle(fast=True)
+    # the reference builds with -march=native: so does the baseline where this host has a compiler
+    native = oracle_build.build_native(tempfile.mkdtemp(prefix="sb_cpu_baseline_"))
+    o = Oracle(path=native) if native else Oracle(fast=True)
+    march = "-march=native (built on this host)" if native else "-march=x86-64-v3 (no compiler on this host)"
     cthr = tau / 2
     info = host_info()
     full_batches = max(1, x.shape[0] // batch)
@@ -193,8 +202,12 @@ def cpu_baseline(x, st, h, mc, batch, tau, dtype, budget_s, min_steps=1, rewire_
                 split[name] += b - a
         return xb.shape[0]
 
-    if warm:
-        step(0, False)  # thread pool, page faults
+    warm_steps = 0
+    if warm:  # thread pool, page faults, caches: five steps, fewer when a step takes seconds
+        tw = time.perf_counter()
+        while warm_steps < 5 and (warm_steps == 0 or time.perf_counter() - tw < 5.0):
+            step(warm_steps, False)
+            warm_steps += 1
     t0 = time.perf_counter()
     samples = steps = 0
     while steps < min_steps or time.perf_counter() - t0 < budget_s:
@@ -208,8 +221,10 @@ def cpu_baseline(x, st, h, mc, batch, tau, dtype, budget_s, min_steps=1, rewire_
     return {"value": samples / dt, "unit": "samples/s", "cores": info["threads_used"], "kind": "port",
             "sample": f"{steps} training step(s) of the same workload (batch {batch}"
                       + (f", rewiring every {rewire_period}th step" if rewire_period else ", no rewiring")
-                      + f"), {dt:.1f} s" + ("" if warm else ", no warm-up step")
-                      + "; C restatement built -O3 -march=x86-64-v3 -ffast-math -fopenmp, forward through numpy's BLAS kernel, one column slice of W per thread",
+                      + f"), {dt:.1f} s after {warm_steps} warm-up step(s)"
+                      + f"; C restatement built -O3 {march} -ffast-math -fopenmp, OMP_PROC_BIND="
+                      + os.environ.get("OMP_PROC_BIND", "") + " OMP_PLACES=" + os.environ.get("OMP_PLACES", "")
+                      + "; forward through numpy's BLAS kernel, one column slice of W per thread",
             "ms_per_step": 1e3 * dt / max(steps, 1),
             "ms_per_step_by_function": {k: 1e3 * v / max(steps, 1) for k, v in split.items()},
             "host": info}

@@ -18,10 +18,11 @@ _P = ctypes.c_void_p
 _L = ctypes.c_long
 
 
-def load(fast=False):
-    name = "libbcpnn_oracle_fast.so" if fast else "libbcpnn_oracle.so"
+def load(fast=False, path=None):
+    """The strict build, the portable fast build, or (path) a library built elsewhere from the same source."""
+    name = path or ("libbcpnn_oracle_fast.so" if fast else "libbcpnn_oracle.so")
     if name not in _LIBS:
-        path = os.path.join(_HERE, name)
+        path = path or os.path.join(_HERE, name)
         if not os.path.exists(path):
             raise RuntimeError(f"{path} missing: run `python oracle/build.py`")
         lib = ctypes.CDLL(path)
@@ -63,9 +64,9 @@ def _chk(a, dtype, name):
 class Oracle:
     """One loaded build of the oracle (strict or fast-math)."""
 
-    def __init__(self, fast=False):
-        self.lib = load(fast)
-        self.fast = fast
+    def __init__(self, fast=False, path=None):
+        self.lib = load(fast, path)
+        self.fast = fast or path is not None
 
     # kernels_openmp.py:6-13
     def update_state(self, state, weights, bias, inputs):

@@ -64,7 +64,9 @@ def _check_layer_at_size(dtype, B, N, H, Mc, density, seed):
     d_act = DeviceArray((B, M), dtype)
     _capi.check(fn("sb_compute_activation")(d_act.ptr, d_x.ptr, d_w.ptr, d_bias.ptr, B, N, H, Mc))
     act = d_act.numpy()
-    assert np.max(np.abs(act - 1.0 / Mc)) <= 10 * tol / Mc
+    e_uniform = float(np.max(np.abs(act - 1.0 / Mc)))  # (|ref| < 1: the suite's metric is the absolute error)
+    record_error("uniform softmax through a constant W", e_uniform, tol)
+    assert e_uniform <= tol
 
     _capi.check(fn("sb_plastic_train_step")(d_w.ptr, d_bias.ptr, d_ci.ptr, d_cj.ptr, d_cij.ptr, d_kbi.ptr,
                                             d_m.ptr, d_x.ptr, d_y.ptr, B, N, H, Mc, tau, khalf, pmin, taubdt,
@@ -107,7 +109,10 @@ def _check_layer_at_size(dtype, B, N, H, Mc, density, seed):
     sample = connected[:: max(1, len(connected) // 2000)]
     got_w = _rows_to_host(_capi, lib, d_w, sample, M, h * Mc, Mc, dtype)
     for k in range(0, len(sample), max(1, len(sample) // 16)):
-        assert np.max(np.abs(got_w[k] - weights_of(sample[k], cols)[1])) <= tol * 30
+        ref_w = weights_of(sample[k], cols)[1]
+        e_w = float(np.max(np.abs(got_w[k] - ref_w) / np.maximum(np.abs(ref_w), 1)))
+        record_error(f"W of hypercolumn {h}, row {sample[k]}", e_w, tol)
+        assert e_w <= tol
     bs = [0, B // 2, B - 1]
     terms = float((x[bs][:, sample].astype(np.float64) @ np.abs(got_w).astype(np.float64)).max())
     terms *= len(connected) / len(sample)
