@@ -67,6 +67,12 @@ struct TrainArgs {
   long tiles_i, tiles_j;
   FastDiv by_panel, by_Mc;  // divisions by tiles_i * panel_cols and by Mc
   unsigned panel_cols;      // tile order: panels of this many tile columns (a power of two), see the kernel
+  // Memory the next launches will read first (the next batch of inputs), or nullptr: a few extra workgroups
+  // touch one element of each of its 128-byte lines, which brings them from HBM into the memory-side cache
+  // (the L2s keep nothing across launches).
+  const void *prefetch;
+  unsigned prefetch_bytes;  // at most 64 MiB
+  unsigned prefetch_lines, prefetch_groups;  // 128-byte lines of the region; workgroups that touch them
 };
 
 // New trace from the old one and the batch's column sum, in the reference's order of operations
@@ -166,8 +172,24 @@ void k_train_fused(TrainArgs<T> a) {
   // The grid has one workgroup per tile; XCD x = blockIdx % 8 holds tiles_of(x) = ntiles / 8 (+1 for
   // x < ntiles % 8) consecutive tiles.
   const unsigned ntiles = (unsigned)a.tiles_i * (unsigned)a.tiles_j;  // < 2^31, checked by the launcher
-  const unsigned xcd = blockIdx.x & 7, rem = ntiles & 7;
-  const unsigned tile = xcd * (ntiles >> 3) + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3);
+  // The first workgroups of the grid (the launcher adds them when there is something to prefetch; a multiple
+  // of 8, so that the tiles keep their XCDs) touch one element
+  // of every 128-byte line of the region, a lane per line, and leave: the lines come from HBM into the
+  // memory-side cache while the tiles compute.  A cold line takes microseconds to arrive, which is why no
+  // tile does this on the side -- its own loads, which return in issue order, would queue behind.
+  if (blockIdx.x < a.prefetch_groups) {  // uniform
+    const __amdgpu_buffer_rsrc_t pwin = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(a.prefetch), 0,
+                                                                          (int)a.prefetch_bytes, 0x00020000);
+    const unsigned first = blockIdx.x * 256 + tid;
+    uint32_t sum = 0;
+    for (unsigned line = first; line < a.prefetch_lines; line += a.prefetch_groups * 256)
+      sum += __builtin_amdgcn_raw_buffer_load_b32(pwin, (int)(line * 128u), 0, 0);
+    asm volatile("" ::"v"(sum));  // (the loads have a consumer)
+    return;
+  }
+  const unsigned wg = blockIdx.x - a.prefetch_groups;
+  const unsigned xcd = wg & 7, rem = ntiles & 7;
+  const unsigned tile = xcd * (ntiles >> 3) + (xcd < rem ? xcd : rem) + (wg >> 3);
   unsigned it, jt;
   if (a.panel_cols == 1) {  // uniform
     jt = a.by_panel.div(tile);

@@ -86,11 +86,13 @@ int launch_softmax(hipStream_t st, T *act, long B, long H, long Mc);
 // Reads the old traces from Ci/Cj and writes the new ones to Ci_next/Cj_next (distinct buffers).
 // W == nullptr: the traces only.
 // w_masked: the caller vouches that W is zero wherever wmask is 0; such entries may then be left alone.
+// prefetch / prefetch_bytes: memory the next launches read first (the next batch), pulled into the
+// memory-side cache by the tiled kernel while it waits for its Cij tiles; optional.
 template <typename T>
 int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci, const T *Cj,
                        T *Ci_next, T *Cj_next, const uint8_t *wmask, int bias_mode, T *bias, T *kbi,
                        long B, long N, long H, long Mc, T taupdt, T cthr, T khalf, T pmin, T taubdt,
-                       bool w_masked);
+                       bool w_masked, const void *prefetch = nullptr, size_t prefetch_bytes = 0);
 // W from the traces as they are, the fused kernel's expression; wmask != nullptr: zero under zero mask bytes
 // (w_masked: the caller vouches that W is zero there already, and such entries are left alone).
 template <typename T>

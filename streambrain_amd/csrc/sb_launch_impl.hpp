@@ -7,6 +7,7 @@
 #include "sb_k_skinny.hpp"
 #include "sb_launch.hpp"
 
+#include <algorithm>
 #include <cstdlib>
 
 namespace sb {
@@ -245,7 +246,7 @@ template <typename T>
 int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, const T *Ci, const T *Cj,
                        T *Ci_next, T *Cj_next, const uint8_t *wmask, int bias_mode, T *bias, T *kbi,
                        long B, long N, long H, long Mc, T taupdt, T cthr, T khalf, T pmin, T taubdt,
-                       bool w_masked) {
+                       bool w_masked, const void *prefetch, size_t prefetch_bytes) {
   constexpr int VW = Real<T>::VW;
   SB_REQUIRE(x && y && Cij && Ci && Cj && Ci_next && Cj_next, "null pointer");  // W may be null: traces only
   SB_REQUIRE(Ci != Ci_next && Cj != Cj_next, "old and new traces must be distinct buffers");
@@ -270,6 +271,16 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   // 8 tile columns beyond that
   a.panel_cols = B * N * (long)sizeof(T) > (2L << 20) ? 8u : 1u;
   a.by_panel = FastDiv::of(a.tiles_i * a.panel_cols); a.by_Mc = FastDiv::of(Mc);
+  // (a region beyond 64 MiB would push more out of the memory-side cache than it brings in)
+  const bool pf = prefetch && prefetch_bytes > 0 && prefetch_bytes <= ((size_t)64 << 20);
+  a.prefetch = pf ? prefetch : nullptr;
+  a.prefetch_bytes = pf ? (unsigned)prefetch_bytes : 0u;
+  a.prefetch_lines = (a.prefetch_bytes + 127) / 128;
+  // a line per thread: what limits a cold fetch is how many misses one CU keeps in flight (a single workgroup
+  // needs 29 us for the 6272 lines of a 128 x 1568 float batch, 25 workgroups on as many CUs finish inside the
+  // tiles' 15 us), so the lines are spread over as many workgroups as there are lines / 256, at most 512
+  // (a multiple of 8: they come first in the grid, and the tiles behind them keep their XCDs)
+  a.prefetch_groups = a.prefetch_lines ? (unsigned)std::min<long>(512, 8 * cdiv(a.prefetch_lines, 8 * 256)) : 0u;
   if (M <= 32) {  // a handful of output units: plain vector arithmetic
     const long rows = skinny_train_rows(M);
     SB_REQUIRE(cdiv(N, rows) < (1L << 31), "too many rows for one launch");
@@ -292,7 +303,8 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   // 16-byte stores of Cij and W need rows that are whole vectors (a vector must not run into the next
   // row); loads are 16-byte accesses for every shape, and neither needs more than element alignment
   const bool vec = M % VW == 0;
-  const dim3 grid((unsigned)(a.tiles_i * a.tiles_j));  // one workgroup per tile
+  // one workgroup per tile (+ the few that prefetch, which the kernel tells apart by their index)
+  const dim3 grid((unsigned)(a.tiles_i * a.tiles_j) + a.prefetch_groups);
   // batch rows per turn of two chunks.  Floats: 32, 18 KiB of LDS per workgroup, so five workgroups share a
   // CU.  Doubles: 16 -- the staging registers of two chunks of 8 rows leave the kernel without spills at four
   // wavefronts per SIMD (1 % faster than 32 at 1568 x 10000, batch 512).
@@ -588,7 +600,7 @@ int launch_copy_pair(hipStream_t st, T *dst1, const T *src1, size_t n1, T *dst2,
   template int launch_softmax<T>(hipStream_t, T *, long, long, long);                                 \
   template int launch_train_fused<T>(hipStream_t, const T *, const T *, T *, T *, const T *, const T *, \
                                      T *, T *, const uint8_t *, int, T *, T *, long, long, long, long, \
-                                     T, T, T, T, T, bool);                                             \
+                                     T, T, T, T, T, bool, const void *, size_t);                                             \
   template int launch_update_bias<T>(hipStream_t, T *, const T *, T, long);                           \
   template int launch_weights_from_traces<T>(hipStream_t, T *, const T *, const T *, const T *,       \
                                              const uint8_t *, T, long, long, long, bool);             \

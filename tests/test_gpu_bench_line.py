@@ -48,6 +48,20 @@ def test_headline_line_short_run():
     assert set(c["ms_per_step_by_function"]) == {"forward_blas", "softmax_numpy", "traces_and_weights", "bias", "mask"}
     assert sum(c["ms_per_step_by_function"].values()) <= c["ms_per_step"] * 1.001
     assert c["host"]["cpu_model"] and c["host"]["threads_used"] >= 1
+    # the passes one by one: each figure follows from its own time and its algorithmic bytes / flops
+    p = b["passes"]
+    n_m = p["shape"]["in_features"] * p["shape"]["hypercolumns"] * p["shape"]["minicolumns"]
+    assert p["weight"]["hbm"]["algorithmic_bytes"] == 2 * 4 * n_m
+    assert p["weight_masked"]["hbm"]["algorithmic_bytes"] == 2 * 4 * n_m + p["shape"]["in_features"] * p["shape"]["hypercolumns"]
+    for name in ("trace", "weight", "weight_masked"):
+        q = p[name]
+        assert q["avg_us"] > 0
+        assert q["hbm"]["GBps"] == pytest.approx(q["hbm"]["algorithmic_bytes"] / (q["avg_us"] * 1e-6) / 1e9, rel=1e-6)
+        assert q["hbm"]["frac_of_hbm_peak"] == pytest.approx(q["hbm"]["GBps"] / 8000.0, rel=1e-9)
+    for name in ("trace", "forward_dense"):
+        q = p[name]
+        assert q["mfma"]["flops"] == 2.0 * p["shape"]["batch"] * n_m
+        assert 0.0 < q["mfma"]["frac_of_mfma_peak"] < 1.0
     o = b["other_configs"]["dense"]
     assert "configs[0]" in o["config"]["workload"] and o["value"] > 0 and 0.0 < o["roofline"]["frac"] < 1.0
     assert o["cpu_baseline"]["value"] > 0
