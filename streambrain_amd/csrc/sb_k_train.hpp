@@ -135,7 +135,8 @@ constexpr int train_waves_per_simd() { return sizeof(T) == 8 ? 4 : (VEC && MB ==
 // MB: mask bytes fetched per vector of VW columns -- 1 when Mc is a multiple of VW (every vector lies
 // inside one hypercolumn), VW otherwise.
 // PRE: Ci_next and Cj_next already hold the new traces (k_trace_sums): no column sums here.
-template <typename T, int KCH, bool VEC, int MB, bool PRE = false>
+// LATE1: the second chunk of the batch is requested only once the first has been staged (see the kernel).
+template <typename T, int KCH, bool VEC, int MB, bool PRE = false, bool LATE1 = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(train_waves_per_simd<T, VEC, MB>())))
 void k_train_fused(TrainArgs<T> a) {
   using R = Real<T>;
@@ -236,12 +237,15 @@ void k_train_fused(TrainArgs<T> a) {
     ynext += KC * M;
     rows_left -= rows;
   };
-  // Only chunk 0 is requested here; chunk 1 follows once chunk 0 sits in LDS (see `chunk`).  The five workgroups
-  // of a CU start together, and what they wait for first is chunk 0: with both chunks requested up front the
-  // CU's first-slab traffic doubles and the first MFMAs start later (1568 x 3000, batch 128: 0.25 us per launch;
-  // the mask bytes and old traces, which only the epilogue needs, likewise wait until the tile is requested:
-  // another 0.1 us).
+  // LATE1 (launches whose workgroups all fit the CUs at once): only chunk 0 is requested here; chunk 1 follows
+  // once chunk 0 sits in LDS (see `chunk`).  The workgroups of a CU then start together, and what they wait for
+  // first is chunk 0: with both chunks requested up front the CU's first-slab traffic doubles and the first
+  // MFMAs start later (1568 x 3000, batch 128: 0.25 us per launch; the mask bytes and old traces, which only
+  // the epilogue needs, likewise wait until the tile is requested: another 0.1 us).  With several rounds of
+  // workgroups a new workgroup starts beside others in full swing, and the earlier request is the better one
+  // (55296 x 20000, batch 256: 4.39 against 4.45 ms).
   request_chunk(std::integral_constant<int, 0>{});
+  if constexpr (!LATE1) request_chunk(std::integral_constant<int, 1>{});
 
   // ---- this lane's share of the tile, in the layout the MFMA leaves it in: wavefront w owns tile rows
   // 16 w .. 16 w + 15 and all 64 columns as four 16 x 16 blocks; the B operand of block c is column
@@ -262,7 +266,8 @@ void k_train_fused(TrainArgs<T> a) {
   }
   const unsigned vstep = rstep * M * ES;  // from acc[..][v] to acc[..][v + 1] (uniform)
 
-  // mask bytes of the lane's synapses: a small, L2-resident array, requested together with the Cij tile
+  // mask bytes of the lane's synapses: a small, L2-resident array, requested up front, or (LATE1) together
+  // with the Cij tile
   const bool masked = a.wmask != nullptr;
   uint32_t mb[4][NG][MB];
   auto request_mask = [&]() {
@@ -290,7 +295,7 @@ void k_train_fused(TrainArgs<T> a) {
   const bool sum_ok = summer && sidx < (sum_i ? N : M);
   const bool writes_bias = !PRE && sum_ok && !sum_i && it == 0 && a.bias_mode == 1;
   // old trace; with PRE the new one, which the same two wavefronts turn into the reciprocals below
-  // (requested together with the Cij tile; unguarded, like every load here)
+  // (requested where the mask bytes are; unguarded, like every load here)
   T cold = T(0), kb = T(1);
   auto request_old_traces = [&]() {
     cold = (PRE ? (sum_i ? a.Ci_next : a.Cj_next) : (sum_i ? a.Ci : a.Cj))[sum_ok ? sidx : 0];
@@ -299,9 +304,15 @@ void k_train_fused(TrainArgs<T> a) {
   T csum = T(0);
 
   T cpre[4][NG][VW];  // Cij tile
-  auto request_tile = [&]() {
+  if constexpr (!LATE1) {
     request_mask();
     request_old_traces();
+  }
+  auto request_tile = [&]() {
+    if constexpr (LATE1) {
+      request_mask();
+      request_old_traces();
+    }
 #pragma unroll
     for (int v = 0; v < 4; v++)
 #pragma unroll
@@ -374,9 +385,9 @@ void k_train_fused(TrainArgs<T> a) {
     // in the first turn of the loop over turns).  The request has to stay behind the staging stores above:
     // moved up by the compiler, ahead of the wait for chunk 0, it would be the early request again -- the
     // uniform branch and the scheduling fence keep it in place.
-    if constexpr (decltype(first)::value == 2) {
+    if constexpr (LATE1 && decltype(first)::value == 2) {
       if (t == 1) request_chunk(std::integral_constant<int, 1>{});
-    } else if constexpr (decltype(first)::value == 1) {
+    } else if constexpr (LATE1 && decltype(first)::value == 1) {
       __builtin_amdgcn_sched_barrier(0);
       request_chunk(std::integral_constant<int, 1>{});
     }
@@ -463,6 +474,30 @@ void k_train_fused(TrainArgs<T> a) {
   constexpr std::integral_constant<int, 0> f0{};
   constexpr std::integral_constant<int, 1> f1{};
   constexpr std::integral_constant<int, 2> f2{};
+  if constexpr (!LATE1) {
+    if constexpr (sizeof(T) == 8) {
+      for (; t < turns; t++) {
+        chunk(set0, no, no, f0);
+        chunk(set1, no, no, f0);
+      }
+      chunk(set0, yes, no, f0);
+      chunk(set1, no, yes, f0);
+    } else {
+      for (; t + 1 < turns; t++) {
+        chunk(set0, no, no, f0);
+        chunk(set1, no, no, f0);
+      }
+      if (turns >= 2) {
+        chunk(set0, no, no, f0);
+        chunk(set1, yes, no, f0);
+        chunk(set0, no, no, f0);
+        chunk(set1, no, yes, f0);
+      } else {
+        chunk(set0, yes, no, f0);
+        chunk(set1, no, yes, f0);
+      }
+    }
+  } else
   if constexpr (sizeof(T) == 8) {
     if (turns >= 2) {
       for (; t < turns; t++) {

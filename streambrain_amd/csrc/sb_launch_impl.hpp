@@ -315,10 +315,15 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   // rows and columns is most of the kernel's vector arithmetic (43 % at 65536 x 100000, batch 1024).
   // From 8 rounds of workgroups on, a small launch computes the new traces once and the tiles read them
   // (timed: 3 % slower at 3 rounds, 3-5 % faster at 8 and 16 rounds, 9 % at 1000).
-  if (vec && one_byte && a.tiles_i * a.tiles_j >= 8 * 5 * device_cu_count()) {
+  const long ntiles = a.tiles_i * a.tiles_j;
+  // one round: every workgroup finds a slot at once (five per CU for floats of whole vectors, else four)
+  const bool one_round = ntiles <= (long)train_waves_per_simd<T, true, 1>() * device_cu_count();
+  if (vec && one_byte && ntiles >= 8 * 5 * device_cu_count()) {
     hipLaunchKernelGGL((k_trace_sums<T>), dim3((unsigned)cdiv(N + M, 256)), dim3(256), 0, st, a);
     hipLaunchKernelGGL((k_train_fused<T, KCH, true, 1, true>), grid, dim3(256), 0, st, a);
-  } else if (vec && one_byte)
+  } else if (vec && one_byte && one_round)
+    hipLaunchKernelGGL((k_train_fused<T, KCH, true, 1, false, true>), grid, dim3(256), 0, st, a);
+  else if (vec && one_byte)
     hipLaunchKernelGGL((k_train_fused<T, KCH, true, 1>), grid, dim3(256), 0, st, a);
   else if (vec)
     hipLaunchKernelGGL((k_train_fused<T, KCH, true, VW>), grid, dim3(256), 0, st, a);
