@@ -8,6 +8,7 @@
   python bench.py --entry-point-rates                                  the per-function C entry points on their own
   python bench.py --passes                                             trace, weight and forward passes one by one
   python bench.py --pmc-summary DIR                                    text summary of rocprofv3 --pmc runs
+  python bench.py --trace-summary DIR                                  per-kernel table of a rocprofv3 kernel trace
 
 Headline workload: the MNIST-shaped 2-layer network, float32, batch 128, 60000 seeded
 synthetic samples; input 784 pixels complementary-coded to 1568 units (~19% nonzero pixels, uniform
@@ -417,7 +418,7 @@ def headline(args):
         "kernels": prof,
         "event_bracket_overhead_us": {"calibrated": bracket_us,
                                       "empty_bracket": run.lib.sb_profile_bracket_overhead_us()},
-        "passes": measure_passes(),
+        "passes": None if args.no_passes else measure_passes(),
         "other_phases": {
             "classifier_layer_train_samples_per_s": cls_samples / cls_dt,
             "classifier_layer_train_first_epoch_samples_per_s": cls_samples / cls_first_dt,
@@ -888,6 +889,22 @@ def _pmc_medians(directory):
     return {k: {c: (len(v), sorted(v)[len(v) // 2]) for c, v in d.items()} for k, d in res.items()}
 
 
+def trace_summary(directory):
+    """Per-kernel table (calls, average / minimum / maximum duration, share of GPU time) from the
+    *_kernel_stats.csv files that `rocprofv3 --kernel-trace --stats --output-format csv` wrote below
+    `directory`."""
+    import csv
+    import glob
+    import re
+    for f in sorted(glob.glob(os.path.join(directory, "**", "*kernel_stats.csv"), recursive=True)):
+        print(f"{'kernel':62s} {'calls':>7s} {'avg us':>9s} {'min us':>9s} {'max us':>9s} {'% of GPU time':>14s}")
+        for r in csv.DictReader(open(f)):
+            name = re.sub(r"^void sb::", "", re.sub(r"\(.*", "", r["Name"]))[:62]
+            print(f"{name:62s} {int(r['Calls']):7d} {float(r['AverageNs']) / 1e3:9.2f} {float(r['MinNs']) / 1e3:9.2f} "
+                  f"{float(r['MaxNs']) / 1e3:9.2f} {float(r['Percentage']):14.2f}")
+    return 0
+
+
 def pmc_summary(directory, calibration=None):
     """Per-kernel medians of the counters in the rocprofv3 --pmc output below `directory` (csv format) as
     text.  With `calibration` (the output of the same counters over `bench.py --copy-calibration`),
@@ -942,9 +959,14 @@ def main():
                          "next to the published peaks)")
     ap.add_argument("--entry-point-rates", action="store_true",
                     help="only time the per-function entry points of the C ABI at the headline layer's shape")
+    ap.add_argument("--no-passes", action="store_true",
+                    help="leave the passes one by one out of the default run (a kernel trace of the run then holds "
+                         "the pipeline's launches only)")
     ap.add_argument("--passes", action="store_true",
                     help="only time the passes of the training step one by one (trace, weight, forward) at the "
                          "headline layer's shape")
+    ap.add_argument("--trace-summary", metavar="DIR",
+                    help="per-kernel table from rocprofv3 --kernel-trace --stats csv output below DIR")
     ap.add_argument("--pmc-summary", metavar="DIR", help="summarise rocprofv3 --pmc csv output below DIR")
     ap.add_argument("--pmc-calibration", metavar="DIR",
                     help="with --pmc-summary: the same counters over `bench.py --copy-calibration`")
@@ -953,6 +975,8 @@ def main():
         print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
               "(the path is not sharded across devices)", file=sys.stderr)
         return 2
+    if args.trace_summary:
+        return trace_summary(args.trace_summary)
     if args.pmc_summary:
         return pmc_summary(args.pmc_summary, args.pmc_calibration)
     if args.copy_calibration:

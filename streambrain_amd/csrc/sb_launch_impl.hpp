@@ -318,7 +318,10 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   const long ntiles = a.tiles_i * a.tiles_j;
   // one round: every workgroup finds a slot at once (five per CU for floats of whole vectors, else four)
   const bool one_round = ntiles <= (long)train_waves_per_simd<T, true, 1>() * device_cu_count();
-  if (vec && one_byte && ntiles >= 8 * 5 * device_cu_count()) {
+  // (doubles, whose ordered additions cost more beside the longer matrix instructions: from 3 rounds of their four
+  // workgroups per CU on -- 1568 x 10000, batch 512: 296 -> 293 us)
+  const long pre_from = sizeof(T) == 8 ? 3 * 4 : 8 * 5;
+  if (vec && one_byte && ntiles >= pre_from * device_cu_count()) {
     hipLaunchKernelGGL((k_trace_sums<T>), dim3((unsigned)cdiv(N + M, 256)), dim3(256), 0, st, a);
     hipLaunchKernelGGL((k_train_fused<T, KCH, true, 1, true>), grid, dim3(256), 0, st, a);
   } else if (vec && one_byte && one_round)
