@@ -8,7 +8,10 @@
 #include <utility>
 #include <mutex>
 #include <random>
+#include <atomic>
+#include <condition_variable>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "../../include/sbhip.h"
@@ -53,6 +56,137 @@ struct Context {
 };
 static Context g_ctx;
 static std::mutex g_ctx_mutex;
+
+// Host -> device copies of caller memory (pageable, as numpy arrays are) through a ring of pinned chunks: the
+// bytes are copied into a pinned chunk by several host threads at once, and the chunk goes to the device with an
+// asynchronous copy while the threads fill the next one.  (One synchronous copy straight from pageable memory
+// runs at about 21 GB/s here; the reference's loader keeps pinned double buffers for the same reason,
+// full_cuda_backend/dataloader.h:36-212.)  The pinned chunks are allocated on first use and kept until
+// sb_shutdown.
+// The host threads that fill a pinned chunk: kThreads - 1 workers that sleep between jobs, plus the caller.
+// The pool lives on the heap and its threads are detached: a process that ends without sb_shutdown must not
+// find joinable threads in a static object.  On release the workers are told to leave; the few bytes of the
+// pool itself stay allocated, so that a worker that wakes late still finds its flags.
+struct CopyPool {
+  static constexpr int kThreads = 8;
+  std::mutex m;
+  std::condition_variable go, done;
+  unsigned long generation = 0;
+  int pending = 0;
+  bool stop = false;
+  char *dst = nullptr;
+  const char *src = nullptr;
+  size_t bytes = 0, piece = 0;
+  void worker(int index) {
+    unsigned long seen = 0;
+    for (;;) {
+      std::unique_lock<std::mutex> lock(m);
+      go.wait(lock, [&] { return stop || generation != seen; });
+      if (stop) return;
+      seen = generation;
+      const size_t at = (size_t)index * piece;
+      char *d = dst;
+      const char *sp = src;
+      const size_t n = at < bytes ? std::min(piece, bytes - at) : 0;
+      lock.unlock();
+      if (n) std::memcpy(d + at, sp + at, n);
+      lock.lock();
+      if (--pending == 0) done.notify_one();
+    }
+  }
+  void start() {
+    for (int k = 1; k < kThreads; k++) std::thread([this, k] { worker(k); }).detach();
+  }
+  // copies bytes in kThreads pieces of whole pages; returns when all of them are done
+  void copy(void *d, const void *sp, size_t n) {
+    if (n < ((size_t)1 << 20)) {
+      std::memcpy(d, sp, n);
+      return;
+    }
+    {
+      std::lock_guard<std::mutex> lock(m);
+      dst = (char *)d;
+      src = (const char *)sp;
+      bytes = n;
+      piece = ((n / kThreads) + 4095) & ~(size_t)4095;
+      pending = kThreads - 1;
+      generation++;
+    }
+    go.notify_all();
+    std::memcpy(d, sp, std::min(piece, n));  // the caller's piece
+    std::unique_lock<std::mutex> lock(m);
+    done.wait(lock, [&] { return pending == 0; });
+  }
+  void leave() {
+    {
+      std::lock_guard<std::mutex> lock(m);
+      stop = true;
+    }
+    go.notify_all();
+  }
+};
+
+struct HostStager {
+  static constexpr int kChunks = 4;
+  static constexpr size_t kChunkBytes = (size_t)8 << 20;
+  void *pinned[kChunks] = {nullptr, nullptr, nullptr, nullptr};
+  hipEvent_t sent[kChunks] = {nullptr, nullptr, nullptr, nullptr};  // the chunk's copy to the device has finished
+  CopyPool *pool = nullptr;
+  hipStream_t copy_stream = nullptr;  // for uploads that run beside the library stream's kernels
+  hipEvent_t uploaded = nullptr, consumed = nullptr;
+  int next = 0;
+  bool ready = false;
+};
+static HostStager g_stager;
+
+static int stager_init() {
+  if (g_stager.ready) return 0;
+  for (int k = 0; k < HostStager::kChunks; k++) {
+    g_allocation_calls += 2;
+    SB_HIP(hipHostMalloc(&g_stager.pinned[k], HostStager::kChunkBytes, hipHostMallocDefault));
+    SB_HIP(hipEventCreateWithFlags(&g_stager.sent[k], hipEventDisableTiming));
+  }
+  g_allocation_calls += 3;
+  SB_HIP(hipStreamCreate(&g_stager.copy_stream));  // (default priority, like the library's stream)
+  SB_HIP(hipEventCreateWithFlags(&g_stager.uploaded, hipEventDisableTiming));
+  SB_HIP(hipEventCreateWithFlags(&g_stager.consumed, hipEventDisableTiming));
+  g_stager.pool = new CopyPool();
+  g_stager.pool->start();
+  g_stager.ready = true;
+  return 0;
+}
+
+static void stager_release() {
+  for (int k = 0; k < HostStager::kChunks; k++) {
+    if (g_stager.pinned[k]) (void)hipHostFree(g_stager.pinned[k]);
+    if (g_stager.sent[k]) (void)hipEventDestroy(g_stager.sent[k]);
+    g_stager.pinned[k] = nullptr;
+    g_stager.sent[k] = nullptr;
+  }
+  if (g_stager.copy_stream) (void)hipStreamDestroy(g_stager.copy_stream);
+  if (g_stager.uploaded) (void)hipEventDestroy(g_stager.uploaded);
+  if (g_stager.consumed) (void)hipEventDestroy(g_stager.consumed);
+  if (g_stager.pool) g_stager.pool->leave();  // (not deleted: see CopyPool)
+  g_stager = HostStager();
+}
+
+// d_dst[0 .. bytes) = h_src[0 .. bytes), ordered on stream `st`.  Returns once h_src has been read (the caller
+// may reuse it); the last chunks may still be on their way to the device, in stream order.
+static int staged_upload(void *d_dst, const void *h_src, size_t bytes, hipStream_t st) {
+  if (bytes == 0) return 0;
+  int rc = stager_init();
+  if (rc) return rc;
+  for (size_t at = 0; at < bytes; at += HostStager::kChunkBytes) {
+    const size_t n = std::min(HostStager::kChunkBytes, bytes - at);
+    const int k = g_stager.next;
+    g_stager.next = (k + 1) % HostStager::kChunks;
+    SB_HIP(hipEventSynchronize(g_stager.sent[k]));  // (an event never recorded counts as finished)
+    g_stager.pool->copy(g_stager.pinned[k], (const char *)h_src + at, n);
+    SB_HIP(hipMemcpyAsync((char *)d_dst + at, g_stager.pinned[k], n, hipMemcpyHostToDevice, st));
+    SB_HIP(hipEventRecord(g_stager.sent[k], st));
+  }
+  return 0;
+}
 
 // Scratch of sb_update_weights_noalloc_f32: the "next" Ci / Cj of the fused kernel for callers that
 // cannot allocate.  Part of the loaded code object, so every GPU the library runs on holds its own copy
@@ -572,15 +706,32 @@ static int net_forward_batches(sb_net *net, const void *h_images, const void *h_
     unsigned long long zero = 0;
     SB_HIP(hipMemcpy(net->d_correct, &zero, sizeof(zero), hipMemcpyHostToDevice));
   }
+  // Inside a chunk the images go up in pieces of whole batches (about 16 MiB) on a copy stream of their own,
+  // through the pinned staging ring; the library's stream waits for a piece's event and works on its batches
+  // while the next piece is on its way.
+  if ((rc = stager_init())) return rc;
+  hipStream_t up = g_stager.copy_stream;
+  long piece = ((long)HostStager::kChunkBytes / (long)(NF * sizeof(T))) / maxB * maxB;
+  if (piece < maxB) piece = maxB;
   for (long c0 = 0; c0 < n && !rc; c0 += chunk) {
     const long rows = (c0 + chunk <= n) ? chunk : n - c0;
-    SB_HIP(hipMemcpy(dX, (const T *)h_images + c0 * NF, (size_t)rows * NF * sizeof(T),
-                     hipMemcpyHostToDevice));
-    if (h_labels)
-      SB_HIP(hipMemcpy(dY, (const T *)h_labels + c0 * NC, (size_t)rows * NC * sizeof(T),
-                       hipMemcpyHostToDevice));
-    if (blocked) rc = launch_gather_rows_blocked<T>(st, (T *)dXB, (T *)nullptr, (const T *)dX, nullptr, rows, NF);
+    if (h_labels) {
+      if ((rc = staged_upload(dY, (const T *)h_labels + c0 * NC, (size_t)rows * NC * sizeof(T), up))) break;
+    }
     for (long lo = 0; lo < rows && !rc; lo += maxB) {
+      if (lo % piece == 0) {  // the piece that starts here
+        const long prows = lo + piece <= rows ? piece : rows - lo;
+        if ((rc = staged_upload((T *)dX + lo * NF, (const T *)h_images + (c0 + lo) * NF,
+                                (size_t)prows * NF * sizeof(T), up)))
+          break;
+        SB_HIP(hipEventRecord(g_stager.uploaded, up));
+        SB_HIP(hipStreamWaitEvent(st, g_stager.uploaded, 0));
+        // (pieces start on multiples of the batch size, which is a multiple of 16 where blocks are used)
+        if (blocked)
+          rc = launch_gather_rows_blocked<T>(st, (T *)dXB + lo * NF, (T *)nullptr, (const T *)dX + lo * NF, nullptr,
+                                             prows, NF);
+        if (rc) break;
+      }
       const long B = (lo + maxB <= rows) ? maxB : rows - lo;
       const T *x = (const T *)dX + lo * NF;
       const T *xb = blocked ? (const T *)dXB + lo * NF : nullptr;
@@ -750,6 +901,7 @@ int sb_shutdown(void) {
   if (g_ctx.mask_nom) SB_HIP(hipFree(g_ctx.mask_nom));
   if (g_ctx.mask_csum) SB_HIP(hipFree(g_ctx.mask_csum));
   if (g_ctx.trace_next) SB_HIP(hipFree(g_ctx.trace_next));
+  stager_release();
   SB_HIP(hipStreamDestroy(g_ctx.stream));
   g_ctx = Context();
   return 0;
@@ -1075,11 +1227,11 @@ int sb_net_set_training_data(sb_net *net, const void *h_images, const void *h_la
   if (rc) return rc;
   const size_t xb = (size_t)n_samples * n_features * net->esize;
   SB_HIP(dev_malloc(&net->X, xb));
-  SB_HIP(hipMemcpy(net->X, h_images, xb, hipMemcpyHostToDevice));
+  if ((rc = staged_upload(net->X, h_images, xb, g_ctx.stream))) return rc;
   if (h_labels) {
     const size_t yb = (size_t)n_samples * n_classes * net->esize;
     SB_HIP(dev_malloc(&net->Y, yb));
-    SB_HIP(hipMemcpy(net->Y, h_labels, yb, hipMemcpyHostToDevice));
+    if ((rc = staged_upload(net->Y, h_labels, yb, g_ctx.stream))) return rc;
   }
   SB_HIP(dev_malloc((void **)&net->d_perm, (size_t)n_samples * sizeof(int64_t)));
   g_allocation_calls++;
