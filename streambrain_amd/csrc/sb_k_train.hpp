@@ -86,29 +86,62 @@ __device__ inline T trace_next(T cold, T sum, const TrainArgs<T> &a) {
   return c > T(0) ? c : T(0);
 }
 
-// The new traces Ci_next, Cj_next (and the regularized bias) on their own, a thread per input or output
-// unit walking the batch in order: what every tile of k_train_fused otherwise repeats for its own 64 rows
-// and 64 columns.  Launched ahead of k_train_fused<.., PRE = true> when a layer has so many tiles that the
-// repetition costs more than a launch.
+// The new traces Ci_next, Cj_next (and the regularized bias) on their own: what every tile of k_train_fused
+// otherwise repeats for its own 64 rows and 64 columns.  Launched ahead of k_train_fused<.., PRE = true> when a
+// layer has so many tiles that the repetition costs more than a launch.  A workgroup takes 64 columns of x or
+// of y.  The sums keep the reference's order (batch row by batch row, one rounded addition each), which is a
+// chain of B dependent additions per column; what the kernel can do is keep the memory latency out of that
+// chain: all 256 threads load the next 64 batch rows (16 independent loads each) into registers while 64 of
+// them add up the previous 64 rows from LDS, where the block was put down ahead of a barrier.  (1568 x 10000
+// doubles, batch 512: 27 -> 12 us, which is the 47 MB of x and y at 4 TB/s; a second block in flight: slower.)
+constexpr int kSumRows = 64;  // batch rows per block
 template <typename T>
 __global__ __launch_bounds__(256) void k_trace_sums(TrainArgs<T> a) {
   using R = Real<T>;
-  const long t = (long)blockIdx.x * 256 + threadIdx.x;
-  const bool is_i = t < a.N;
-  const long idx = is_i ? t : t - a.N;
-  if (!is_i && idx >= a.M) return;
-  const T *p = (is_i ? a.x : a.y) + idx;
-  const long stride = is_i ? a.N : a.M;
+  __shared__ T block[2][kSumRows][64];
+  const int tid = threadIdx.x, col = tid & 63, sub = tid >> 6;  // thread (sub, col) loads rows sub, sub + 4, ..
+  const long groups_i = (a.N + 63) / 64;
+  const bool is_i = (long)blockIdx.x < groups_i;
+  const long width = is_i ? a.N : a.M;
+  const long idx = (is_i ? (long)blockIdx.x : (long)blockIdx.x - groups_i) * 64 + col;
+  const T *const src = is_i ? a.x : a.y;
+  constexpr int PER = kSumRows / 4;  // loads per thread and block
+  const unsigned es = sizeof(T);
+  T v[PER];
+  auto request = [&](long b0) {
+    // a window over the block's rows (below 2 GiB: the launcher checks 64 rows of the wider matrix); rows
+    // past the batch lie outside it and read zero, like the columns past the matrix
+    const long rows = a.B - b0 < kSumRows ? a.B - b0 : kSumRows;
+    const BufferWindow<T> win(uniform_pointer(src + b0 * width),
+                              typename BufferWindow<T>::Bytes{(unsigned)(rows * width * es)});
+#pragma unroll
+    for (int k = 0; k < PER; k++) {
+      const long r = sub + 4 * k;
+      T one[1];
+      win.template load_n<1>(one, idx < width ? (unsigned)((r * width + idx) * es) : BufferWindow<T>::kOutside);
+      v[k] = one[0];
+    }
+  };
+  request(0);
   T sum = T(0);
-  long b = 0;
-  for (; b + 16 <= a.B; b += 16) {  // 16 loads in flight, then the ordered additions
-    T v[16];
+  int buf = 0;
+  for (long b0 = 0; b0 < a.B; b0 += kSumRows, buf ^= 1) {
 #pragma unroll
-    for (int k = 0; k < 16; k++) v[k] = p[(b + k) * stride];
+    for (int k = 0; k < PER; k++) block[buf][sub + 4 * k][col] = v[k];
+    if (b0 + kSumRows < a.B) request(b0 + kSumRows);  // (uniform) in flight during the additions below
+    __syncthreads();  // the block is there; the buffer written next time round was read before this barrier
+    if (sub == 0) {
+      constexpr int U = 8;
+      for (int r = 0; r < kSumRows; r += U) {
+        T w[U];
 #pragma unroll
-    for (int k = 0; k < 16; k++) sum = R::add(sum, v[k]);
+        for (int k = 0; k < U; k++) w[k] = block[buf][r + k][col];
+#pragma unroll
+        for (int k = 0; k < U; k++) sum = R::add(sum, w[k]);  // (zeros past the batch change nothing)
+      }
+    }
   }
-  for (; b < a.B; b++) sum = R::add(sum, p[b * stride]);
+  if (sub != 0 || idx >= width) return;
   const T cnew = trace_next<T>((is_i ? a.Ci : a.Cj)[idx], sum, a);
   if (is_i) {
     a.Ci_next[idx] = cnew;

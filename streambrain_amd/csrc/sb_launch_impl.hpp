@@ -313,16 +313,16 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   ProfScope prof_(st, K_TRAIN_FUSED);
   // Every tile adds up the batch's x and y columns for its own rows and columns, which with many tile
   // rows and columns is most of the kernel's vector arithmetic (43 % at 65536 x 100000, batch 1024).
-  // From 8 rounds of workgroups on, a small launch computes the new traces once and the tiles read them
-  // (timed: 3 % slower at 3 rounds, 3-5 % faster at 8 and 16 rounds, 9 % at 1000).
+  // From one and a half rounds of workgroups on (floats; doubles: two and a half), a small launch computes the
+  // new traces once and the tiles read them.  Timed, 4096 inputs, batch 128, floats, with / without that
+  // launch: 23.7 / 22.5 us at 1.05 rounds, 29.3 / 29.9 at 1.5, 34.6 / 35.6 at 2, 45.5 / 48.5 at 3, 67.1 / 69.2
+  // at 5; doubles: 48.1 / 47.3 at 1.6 rounds, 55.8 / 54.3 at 2, 110.3 / 113.7 at 2.5.
   const long ntiles = a.tiles_i * a.tiles_j;
   // one round: every workgroup finds a slot at once (five per CU for floats of whole vectors, else four)
   const bool one_round = ntiles <= (long)train_waves_per_simd<T, true, 1>() * device_cu_count();
-  // (doubles, whose ordered additions cost more beside the longer matrix instructions: from 3 rounds of their four
-  // workgroups per CU on -- 1568 x 10000, batch 512: 296 -> 293 us)
-  const long pre_from = sizeof(T) == 8 ? 3 * 4 : 8 * 5;
-  if (vec && one_byte && ntiles >= pre_from * device_cu_count()) {
-    hipLaunchKernelGGL((k_trace_sums<T>), dim3((unsigned)cdiv(N + M, 256)), dim3(256), 0, st, a);
+  const long pre_from = sizeof(T) == 8 ? 5 * 4 : 3 * 5;  // in half workgroups per CU
+  if (vec && one_byte && 2 * ntiles >= pre_from * device_cu_count()) {
+    hipLaunchKernelGGL((k_trace_sums<T>), dim3((unsigned)(cdiv(N, 64) + cdiv(M, 64))), dim3(256), 0, st, a);
     hipLaunchKernelGGL((k_train_fused<T, KCH, true, 1, true>), grid, dim3(256), 0, st, a);
   } else if (vec && one_byte && one_round)
     hipLaunchKernelGGL((k_train_fused<T, KCH, true, 1, false, true>), grid, dim3(256), 0, st, a);

@@ -168,8 +168,9 @@ def _trace_problem(rng, B, N, M, dtype):
                                            # columns; 11 and 8 tile columns (narrow and no last panel)
                                            (64, 8300, 700), (48, 5600, 512),
                                            # 150 x 141 tiles: the traces come from their own launch (one
-                                           # turn of two chunks; two turns; a loop turn ahead of them)
-                                           (8, 9600, 9000), (40, 9600, 9000), (72, 7040, 6016)])
+                                           # turn of two chunks; two turns; a loop turn ahead of them; that
+                                           # launch's blocks of 64 batch rows: a ragged second, four)
+                                           (8, 9600, 9000), (40, 9600, 9000), (72, 7040, 6016), (200, 7040, 6016)])
 def test_update_weights(k, oracle, dtype, B, N, M):
     rng = np.random.default_rng(B + 2 * N + 3 * M)
     x, y, Ci, Cj, Cij = _trace_problem(rng, B, N, M, dtype)
