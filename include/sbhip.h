@@ -306,7 +306,9 @@ int sb_net_layer_train_finalize(sb_net *net, int layer);
  * [0, sb_profile_kernels()), the summed elapsed time and the number of launches.  The reference has no
  * counterpart (it times whole runs with time.time(), train.py:181-193).  The sums are raw bracket times:
  * a bracket adds a few microseconds of its own to a short kernel (compare the bracketed sum of a run
- * with its unbracketed wall time to calibrate). */
+ * with its unbracketed wall time to calibrate).  The fused training launch is the exception: its events ride on
+ * the launch itself (sb_profile_kernel_carried), except under rocprofv3, where they would read long and the
+ * launch is bracketed like the others. */
 int sb_profile_start(void);
 int sb_profile_stop(void);
 int sb_profile_kernels(void);
@@ -314,6 +316,10 @@ int sb_profile_kernels(void);
  * what a bracket adds to a launch. */
 double sb_profile_bracket_overhead_us(void);
 const char *sb_profile_kernel_name(int kernel);
+/* 1 when the launches of that kernel carry their events themselves (stamped with the dispatch's own begin and
+ * end, as a kernel trace reports them: nothing to subtract), 0 when the events are records on the stream
+ * around the launches (which add what sb_profile_bracket_overhead_us bounds). */
+int sb_profile_kernel_carried(int kernel);
 int sb_profile_get(int kernel, double *total_ms, long *launches);
 
 /* Matrix-core probe for the achievable-peak record of bench.py: `workgroups` workgroups of four wavefronts

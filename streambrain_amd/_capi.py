@@ -77,6 +77,7 @@ _PLAIN_SIGS = {
 }
 _RESTYPES = {"sb_last_error": ctypes.c_char_p, "sb_stream": _P, "sb_allocation_calls": _L}
 _OTHER_SIGS = {"sb_profile_kernel_name": ([_I], ctypes.c_char_p),
+               "sb_profile_kernel_carried": ([_I], _I),
                "sb_profile_bracket_overhead_us": ([], _D)}
 
 

@@ -35,11 +35,21 @@ enum KernelId {
 };
 const char *kernel_name(int id);
 struct ProfScope {
-  ProfScope(hipStream_t st, int id);
+  // carried = false: the scope records an event on the stream ahead of the launches and one behind them.
+  // carried = true: the launches themselves carry the events (hipExtLaunchKernelGGL takes a start and a stop
+  // event and stamps them with the dispatch's own begin and end, which is what a kernel trace reports): the
+  // scope records nothing, the caller passes start() to its first launch and stop() to its last.
+  ProfScope(hipStream_t st, int id, bool carried = false);
   ~ProfScope();
+  bool carries() const { return slot_ >= 0 && carried_; }  // the caller's launches take start() and stop()
+  hipEvent_t start() const;
+  hipEvent_t stop() const;
   hipStream_t st_;
   int slot_;
+  bool carried_;
 };
+// whether the durations recorded for kernel index `id` come from events carried by the launches
+bool prof_carried(int id);
 
 void set_error(const std::string &msg);
 int hip_fail(hipError_t e, const char *what, const char *file, int line);

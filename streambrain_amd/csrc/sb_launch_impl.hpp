@@ -8,6 +8,7 @@
 #include "sb_launch.hpp"
 
 #include <algorithm>
+#include <hip/hip_ext.h>
 #include <cstdlib>
 
 namespace sb {
@@ -284,14 +285,18 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   if (M <= 32) {  // a handful of output units: plain vector arithmetic
     const long rows = skinny_train_rows(M);
     SB_REQUIRE(cdiv(N, rows) < (1L << 31), "too many rows for one launch");
-    ProfScope prof_(st, K_TRAIN_FUSED);
+    ProfScope prof_(st, K_TRAIN_FUSED, true);
     // batch rows staged per chunk (see the kernel)
     long bc = kSkinnyLoads * (256 / rows) < kSkinnyLoads * (256 / M) ? kSkinnyLoads * (256 / rows) : kSkinnyLoads * (256 / M);
     if (bc > kSkinnyStage / (rows + M)) bc = kSkinnyStage / (rows + M);
     if (bc > ((1L << 31) - 1) / (N * (long)sizeof(T))) bc = ((1L << 31) - 1) / (N * (long)sizeof(T));
     if (bc > B) bc = B;
     SB_REQUIRE(bc >= 1, "layer too wide for the small-output training kernel");
-    hipLaunchKernelGGL((k_train_skinny<T>), dim3((unsigned)cdiv(N, rows)), dim3(256), 0, st, a, (int)bc);
+    if (prof_.carries())
+      hipExtLaunchKernelGGL((k_train_skinny<T>), dim3((unsigned)cdiv(N, rows)), dim3(256), 0, st, prof_.start(),
+                            prof_.stop(), 0, a, (int)bc);
+    else
+      hipLaunchKernelGGL((k_train_skinny<T>), dim3((unsigned)cdiv(N, rows)), dim3(256), 0, st, a, (int)bc);
     SB_LAUNCH_CHECK();
     return 0;
   }
@@ -310,7 +315,15 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   // wavefronts per SIMD (1 % faster than 32 at 1568 x 10000, batch 512).
   constexpr int KCH = sizeof(T) == 8 ? 16 : 32;
   const bool one_byte = Mc % VW == 0;  // every vector of VW columns lies inside one hypercolumn
-  ProfScope prof_(st, K_TRAIN_FUSED);
+  ProfScope prof_(st, K_TRAIN_FUSED, true);
+  // one launch, or the sum launch and the tile launch, with the profile's events riding on them
+  auto launch = [&](auto kernel, dim3 g, bool first, bool last) {
+    if (prof_.carries())
+      hipExtLaunchKernelGGL(kernel, g, dim3(256), 0, st, first ? prof_.start() : nullptr,
+                            last ? prof_.stop() : nullptr, 0, a);
+    else
+      hipLaunchKernelGGL(kernel, g, dim3(256), 0, st, a);
+  };
   // Every tile adds up the batch's x and y columns for its own rows and columns, which with many tile
   // rows and columns is most of the kernel's vector arithmetic (43 % at 65536 x 100000, batch 1024).
   // From one and a half rounds of workgroups on (floats; doubles: two and a half), a small launch computes the
@@ -322,18 +335,18 @@ int launch_train_fused(hipStream_t st, const T *x, const T *y, T *Cij, T *W, con
   const bool one_round = ntiles <= (long)train_waves_per_simd<T, true, 1>() * device_cu_count();
   const long pre_from = sizeof(T) == 8 ? 5 * 4 : 3 * 5;  // in half workgroups per CU
   if (vec && one_byte && 2 * ntiles >= pre_from * device_cu_count()) {
-    hipLaunchKernelGGL((k_trace_sums<T>), dim3((unsigned)(cdiv(N, 64) + cdiv(M, 64))), dim3(256), 0, st, a);
-    hipLaunchKernelGGL((k_train_fused<T, KCH, true, 1, true>), grid, dim3(256), 0, st, a);
+    launch(k_trace_sums<T>, dim3((unsigned)(cdiv(N, 64) + cdiv(M, 64))), true, false);
+    launch(k_train_fused<T, KCH, true, 1, true>, grid, false, true);
   } else if (vec && one_byte && one_round)
-    hipLaunchKernelGGL((k_train_fused<T, KCH, true, 1, false, true>), grid, dim3(256), 0, st, a);
+    launch(k_train_fused<T, KCH, true, 1, false, true>, grid, true, true);
   else if (vec && one_byte)
-    hipLaunchKernelGGL((k_train_fused<T, KCH, true, 1>), grid, dim3(256), 0, st, a);
+    launch(k_train_fused<T, KCH, true, 1>, grid, true, true);
   else if (vec)
-    hipLaunchKernelGGL((k_train_fused<T, KCH, true, VW>), grid, dim3(256), 0, st, a);
+    launch(k_train_fused<T, KCH, true, VW>, grid, true, true);
   else if (one_byte)
-    hipLaunchKernelGGL((k_train_fused<T, KCH, false, 1>), grid, dim3(256), 0, st, a);
+    launch(k_train_fused<T, KCH, false, 1>, grid, true, true);
   else
-    hipLaunchKernelGGL((k_train_fused<T, KCH, false, VW>), grid, dim3(256), 0, st, a);
+    launch(k_train_fused<T, KCH, false, VW>, grid, true, true);
   SB_LAUNCH_CHECK();
   return 0;
 }

@@ -225,17 +225,25 @@ static hipEvent_t prof_event() {
   return e;
 }
 
-ProfScope::ProfScope(hipStream_t st, int id) : st_(st), slot_(-1) {
+// Under rocprofv3 (which sets ROCPROF_OUTPUT_PATH for the program it runs) the dispatch timestamps belong to the
+// profiler and events carried by a launch read long (29 us for a 16 us kernel): the scopes bracket then.
+static bool g_prof_carry = true;
+ProfScope::ProfScope(hipStream_t st, int id, bool carried)
+    : st_(st), slot_(-1), carried_(carried && g_prof_carry) {
+  carried = carried_;
   if (!g_prof_on) return;
   ProfRecord r{id, prof_event(), prof_event()};
   if (!r.start || !r.stop) return;
-  (void)hipEventRecord(r.start, st);
+  if (!carried) (void)hipEventRecord(r.start, st);
   g_prof_records.push_back(r);
   slot_ = (int)g_prof_records.size() - 1;
 }
 ProfScope::~ProfScope() {
-  if (slot_ >= 0) (void)hipEventRecord(g_prof_records[slot_].stop, st_);
+  if (slot_ >= 0 && !carried_) (void)hipEventRecord(g_prof_records[slot_].stop, st_);
 }
+hipEvent_t ProfScope::start() const { return slot_ >= 0 ? g_prof_records[slot_].start : nullptr; }
+hipEvent_t ProfScope::stop() const { return slot_ >= 0 ? g_prof_records[slot_].stop : nullptr; }
+bool prof_carried(int id) { return g_prof_carry && id == K_TRAIN_FUSED; }
 
 static int require_ready() {
   if (!g_ctx.ready) {
@@ -1338,6 +1346,7 @@ int sb_profile_start(void) {
     g_prof_ms[k] = 0;
     g_prof_launches[k] = 0;
   }
+  g_prof_carry = std::getenv("ROCPROF_OUTPUT_PATH") == nullptr;
   // what a bracket costs at most: median elapsed time of event pairs with nothing in between (reported
   // by sb_profile_bracket_overhead_us; the per-kernel sums stay raw)
   {
@@ -1386,6 +1395,8 @@ int sb_profile_kernels(void) { return K_COUNT; }
 double sb_profile_bracket_overhead_us(void) { return 1e3 * g_prof_overhead_ms; }
 
 const char *sb_profile_kernel_name(int kernel) { return kernel_name(kernel); }
+
+int sb_profile_kernel_carried(int kernel) { return kernel >= 0 && kernel < K_COUNT && prof_carried(kernel) ? 1 : 0; }
 
 int sb_profile_get(int kernel, double *total_ms, long *launches) {
   SB_REQUIRE(kernel >= 0 && kernel < K_COUNT && total_ms && launches, "bad argument");
