@@ -36,6 +36,10 @@ def test_headline_line_short_run():
     assert r["bound"] == "hbm" and r["unit"] == "GB/s" and r["peak"] == 8000.0
     assert r["frac"] == pytest.approx(r["achieved"] / r["peak"], rel=1e-9) and 0.0 < r["frac"] < 1.0
     assert r["achieved"] == pytest.approx(r["algorithmic_bytes_per_launch"] / (r["avg_launch_us"] * 1e-6) / 1e9, rel=1e-6)
+    # the dominant kernel's duration comes from events its launches carry (dispatch begin to end): nothing subtracted
+    k = b["kernels"]["train_fused"]
+    assert k["events"] == "carried" and k["avg_us"] == k["raw_avg_us"] == r["avg_launch_us"]
+    assert b["kernels"]["forward"]["events"] == "bracket" and b["kernels"]["forward"]["avg_us"] < b["kernels"]["forward"]["raw_avg_us"]
     # the counter summary in profiles/ belongs to the kernel sources of this tree
     assert r["traffic"] is not None, r["traffic_note"]
     assert 0.5 * r["algorithmic_bytes_per_launch"] < r["traffic"] < 2 * r["algorithmic_bytes_per_launch"]
