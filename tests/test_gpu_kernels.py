@@ -55,7 +55,7 @@ def test_update_state(k, oracle, dtype, B, N, M):
 
 # ------------------------------------------------------------- forward over the connected rows only
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("rows,cols", [(1, 1), (16, 5), (37, 300), (128, 1568)])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (16, 5), (37, 300), (50, 302), (128, 1568)])
 def test_rows_in_blocks(k, dtype, rows, cols):
     rng = np.random.default_rng(rows + cols)
     a = rng.random((rows, cols)).astype(dtype)
