@@ -11,6 +11,7 @@
 #include <atomic>
 #include <condition_variable>
 #include <string>
+#include <system_error>
 #include <thread>
 #include <vector>
 
@@ -94,12 +95,20 @@ struct CopyPool {
       if (--pending == 0) done.notify_one();
     }
   }
+  int workers = 0;  // started; a thread the system refuses is done without
   void start() {
-    for (int k = 1; k < kThreads; k++) std::thread([this, k] { worker(k); }).detach();
+    for (int k = 1; k < kThreads; k++) {
+      try {
+        std::thread([this, k] { worker(k); }).detach();
+      } catch (const std::system_error &) {
+        break;
+      }
+      workers = k;
+    }
   }
-  // copies bytes in kThreads pieces of whole pages; returns when all of them are done
+  // copies bytes in pieces of whole pages, one per thread; returns when all of them are done
   void copy(void *d, const void *sp, size_t n) {
-    if (n < ((size_t)1 << 20)) {
+    if (n < ((size_t)1 << 20) || workers == 0) {
       std::memcpy(d, sp, n);
       return;
     }
@@ -108,8 +117,8 @@ struct CopyPool {
       dst = (char *)d;
       src = (const char *)sp;
       bytes = n;
-      piece = ((n / kThreads) + 4095) & ~(size_t)4095;
-      pending = kThreads - 1;
+      piece = ((n / (size_t)(workers + 1)) + 4095) & ~(size_t)4095;
+      pending = workers;
       generation++;
     }
     go.notify_all();
