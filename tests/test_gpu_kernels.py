@@ -91,7 +91,11 @@ def test_mask_rows(k, N, H, density):
                                               (20, 6000, 2, 64, 0.5),  # lists longer than one LDS segment
                                               # many tiles: 32 and 64 batch rows per workgroup, ragged
                                               (1000, 300, 32, 100, 0.2), (2030, 200, 64, 100, 0.3),
-                                              (12, 40, 2, 224, 0.5)])
+                                              (12, 40, 2, 224, 0.5),
+                                              # many hypercolumns: narrow (12 columns) and full (128) ones, a
+                                              # ragged batch, lists longer than one LDS segment
+                                              (130, 300, 260, 12, 0.3), (256, 400, 140, 128, 0.2),
+                                              (128, 5000, 260, 12, 0.5)])
 @pytest.mark.parametrize("blocked", [False, True])
 def test_compute_activation_rows(k, oracle, dtype, B, N, H, Mc, density, blocked):
     """The row-list forward kernel against the dense reference computation on the masked weights."""
