@@ -264,7 +264,7 @@ def test_weights_masked_from_counters(k, oracle, dtype, N, H, Mc, density):
 def test_weight_logarithm_f64_within_two_ulp(k):
     """The double-precision weight pass evaluates its logarithm with a short routine of the library's own
     (argument reduction, degree-7 polynomial, hardware reciprocal) instead of the runtime's.  With Ci = Cj = 1 a
-    weight is log(max(Cij, cthr^4)): arguments over 60 binades, around 1 (where the result cancels to nearly
+    weight is log(max(Cij, cthr^4)): arguments over 60 binades, close to 1 (where the result cancels to nearly
     nothing), at and around powers of two and the reduction's switch at sqrt(1/2), checked against an 80-bit
     logarithm rounded to double.  Measured: 0.75 ulp on the CPU restatement of the same routine."""
     rng = np.random.default_rng(99)
