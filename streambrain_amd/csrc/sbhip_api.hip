@@ -5,8 +5,10 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <exception>
 #include <utility>
 #include <mutex>
+#include <new>
 #include <random>
 #include <atomic>
 #include <condition_variable>
@@ -873,6 +875,20 @@ static int layer_state(sb_net *net, int layer, const char *name, StateRef &out) 
   return 0;
 }
 
+// The C entry points whose host-side work allocates (vectors sized by the layer, the network object) run it
+// through this: an exception must not cross the C boundary.
+template <typename F>
+static int no_throw(const char *where, F &&body) {
+  try {
+    return body();
+  } catch (const std::bad_alloc &) {
+    set_error(std::string(where) + ": out of host memory");
+  } catch (const std::exception &e) {
+    set_error(std::string(where) + ": " + e.what());
+  }
+  return SB_ERR_STATE;
+}
+
 }  // namespace sb
 
 using namespace sb;
@@ -1107,7 +1123,11 @@ int sb_net_create(sb_net **net, int dtype) {
   SB_READY();
   SB_REQUIRE(net, "null pointer");
   SB_REQUIRE(dtype == SB_F32 || dtype == SB_F64, "dtype must be SB_F32 or SB_F64");
-  sb_net *n = new sb_net();
+  sb_net *n = new (std::nothrow) sb_net();
+  if (!n) {
+    set_error("sb_net_create: out of host memory");
+    return SB_ERR_STATE;
+  }
   n->dtype = dtype;
   n->esize = dtype == SB_F32 ? 4 : 8;
   hipError_t e = dev_malloc((void **)&n->d_correct, sizeof(unsigned long long));
@@ -1176,15 +1196,19 @@ static int add_layer(sb_net *net, bool plastic, long n_inputs, long H, long Mc, 
 
 int sb_net_add_dense_layer(sb_net *net, long n_inputs, long hypercolumns, long minicolumns,
                            double taupdt, double initial_Ci, double initial_Cj, double initial_Cij) {
-  return add_layer(net, false, n_inputs, hypercolumns, minicolumns, taupdt, 0, 0, 0, initial_Ci,
-                   initial_Cj, initial_Cij);
+  return no_throw("sb_net_add_dense_layer", [&] {
+    return add_layer(net, false, n_inputs, hypercolumns, minicolumns, taupdt, 0, 0, 0, initial_Ci, initial_Cj,
+                     initial_Cij);
+  });
 }
 
 int sb_net_add_plastic_layer(sb_net *net, long n_inputs, long hypercolumns, long minicolumns,
                              double taupdt, double pmin, double khalf, double taubdt,
                              double initial_Ci, double initial_Cj, double initial_Cij) {
-  return add_layer(net, true, n_inputs, hypercolumns, minicolumns, taupdt, pmin, khalf, taubdt,
-                   initial_Ci, initial_Cj, initial_Cij);
+  return no_throw("sb_net_add_plastic_layer", [&] {
+    return add_layer(net, true, n_inputs, hypercolumns, minicolumns, taupdt, pmin, khalf, taubdt, initial_Ci,
+                     initial_Cj, initial_Cij);
+  });
 }
 
 int sb_net_set_layer_state(sb_net *net, int layer, const char *name, const void *h_src, size_t bytes) {
@@ -1200,8 +1224,10 @@ int sb_net_set_layer_state(sb_net *net, int layer, const char *name, const void 
   Layer &L = net->layers[layer];
   if (s.ptr == L.W) L.w_masked = false, L.w_unchecked = true;
   if (s.ptr == L.wmask)
-    return net->dtype == SB_F32 ? layer_mask_replaced<float>(L, (const uint8_t *)h_src)
-                                : layer_mask_replaced<double>(L, (const uint8_t *)h_src);
+    return no_throw("sb_net_set_layer_state", [&] {
+      return net->dtype == SB_F32 ? layer_mask_replaced<float>(L, (const uint8_t *)h_src)
+                                  : layer_mask_replaced<double>(L, (const uint8_t *)h_src);
+    });
   return 0;
 }
 
@@ -1221,8 +1247,10 @@ int sb_net_randomize_layer(sb_net *net, int layer, uint64_t seed, double density
   SB_REQUIRE(layer >= 0 && layer < (int)net->layers.size(), "layer index out of range");
   SB_REQUIRE(density >= 0.0, "density must be non-negative");
   SB_HIP(hipStreamSynchronize(g_ctx.stream));
-  return net->dtype == SB_F32 ? net_randomize_layer<float>(net, layer, seed, density)
-                              : net_randomize_layer<double>(net, layer, seed, density);
+  return no_throw("sb_net_randomize_layer", [&] {
+    return net->dtype == SB_F32 ? net_randomize_layer<float>(net, layer, seed, density)
+                                : net_randomize_layer<double>(net, layer, seed, density);
+  });
 }
 
 int sb_net_set_frozen_cache_limit(sb_net *net, size_t bytes) {
