@@ -65,3 +65,20 @@ def test_pmc_summary_scales_by_the_copy_calibration(tmp_path):
     want = (14147.0 * 2 + 20310.0) * 1024
     line = [ln for ln in out.splitlines() if ln.startswith("traffic_bytes_per_launch:")]
     assert line and abs(float(line[0].split(":")[1]) - want) < 1.0
+
+
+def test_bracket_calibration_leaves_carried_events_alone():
+    """Kernels whose events ride on the launch keep their measured duration; the others lose the per-bracket
+    cost that follows from the bracketed and the unbracketed pass, capped at an empty bracket's time."""
+    sys.path.insert(0, ROOT)
+    import bench
+    kernels = {"train_fused": {"launches": 100, "raw_avg_us": 16.0, "events": "carried"},
+               "forward": {"launches": 100, "raw_avg_us": 9.0, "events": "bracket"}}
+    raw_ms = (100 * 16.0 + 100 * 9.0) / 1e3
+    # unbracketed: 100 steps of 22.5 us -> the 100 brackets added 2.5 us each
+    us = bench.calibrate_brackets(kernels, raw_ms, 100, 100 * 22.5e-6, upper_us=4.4)
+    assert abs(us - 2.5) < 1e-9
+    assert kernels["train_fused"]["avg_us"] == 16.0 and abs(kernels["forward"]["avg_us"] - 6.5) < 1e-9
+    # a profiler that slows the bracketed pass down: no more than an empty bracket is taken off
+    us = bench.calibrate_brackets(kernels, raw_ms + 1.0, 100, 100 * 22.5e-6, upper_us=4.4)
+    assert us == 4.4 and abs(kernels["forward"]["avg_us"] - 4.6) < 1e-9
