@@ -168,9 +168,10 @@ def _trace_problem(rng, B, N, M, dtype):
 
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("B,N,M", SHAPES + [(128, 1568, 3000), (5, 130, 70), (1024, 64, 64),
-                                           # batch of x above 2 MiB: tiles walked in panels of 8 tile
-                                           # columns; 11 and 8 tile columns (narrow and no last panel)
-                                           (64, 8300, 700), (48, 5600, 512),
+                                           # batch of x above 2 MiB: tiles walked in panels of 16 tile
+                                           # columns (11 and 8 tile columns: one narrow panel; 18: a full one
+                                           # and a rest), of 8 for batches beyond 512 rows (10 tile columns)
+                                           (64, 8300, 700), (48, 5600, 512), (64, 8300, 1100), (520, 1100, 600),
                                            # 150 x 141 tiles: the traces come from their own launch (one
                                            # turn of two chunks; two turns; a loop turn ahead of them; that
                                            # launch's blocks of 64 batch rows: a ragged second, four)
