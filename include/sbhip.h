@@ -272,7 +272,9 @@ int sb_net_train_batches(sb_net *net, int layer, long maximal_batch_size,
 
 /* Network.evaluate (_cpu_base_backend.py:205-245): forward through every layer, count rows whose
  * argmax equals the label's argmax.  Synchronous.  h_pred (may be NULL) receives the predicted
- * class per row. */
+ * class per row.  The host arrays go up in pieces through pinned staging buffers while earlier pieces are
+ * computed; the device buffers of a chunk of the set (at most about 2 x 256 MiB of images, plus labels and
+ * predictions) are kept with the network for the next call and released by sb_net_destroy. */
 int sb_net_evaluate(sb_net *net, const void *h_images, const void *h_labels, long n_samples,
                     long n_features, long n_classes, long maximal_batch_size, int64_t *correct,
                     int64_t *total, int32_t *h_pred);
