@@ -187,6 +187,8 @@ static int forward_rows_variant(hipStream_t st, ForwardRowsArgs<T> a) {
     if (rb == 4) {
     } else if (rb == 2)
       hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 2, true, LW>), g, blk, 0, st, a);
+    else if (a.cap <= 256)  // short lists: a segment of 256 entries (see the kernel)
+      hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 1, true, LW, 256>), g, blk, 0, st, a);
     else
       hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 1, true, LW>), g, blk, 0, st, a);
   } else {
@@ -196,6 +198,8 @@ static int forward_rows_variant(hipStream_t st, ForwardRowsArgs<T> a) {
     if (rb == 4) {
     } else if (rb == 2)
       hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 2, false, LW>), g, blk, 0, st, a);
+    else if (a.cap <= 256)
+      hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 1, false, LW, 256>), g, blk, 0, st, a);
     else
       hipLaunchKernelGGL((k_forward_rows<T, NG, NW, 1, false, LW>), g, blk, 0, st, a);
   }
