@@ -74,12 +74,16 @@ struct ForwardBias {
 // tail: with TAIL, the tile's last four columns (tail_col0 .. +3 of the tile) as the 4x4 products of
 // Real<T>::mfma_4x4 leave them: element v of lane (p, q) is row 4 (p/4) + v, column p % 4, summed over the
 // reduction indices of q only.
-template <typename T, int NG, bool FUSE, int NWAVES, int LW, bool TAIL = false>
+// NT: tiles of LDS the partial sums go through.  NWAVES / 2: the two-step hand-over described below.  NWAVES: every
+// wavefront puts its partial tile down and the row-wise pass adds up all of them -- twice the LDS, one barrier
+// and one dependent round trip through LDS less (for the kernels whose time is a chain of latencies).
+template <typename T, int NG, bool FUSE, int NWAVES, int LW, bool TAIL = false, int NT = NWAVES / 2>
 __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&acc)[NG][Real<T>::VW],
                                                const T (&bv)[ForwardBias<T, NG, NWAVES>::PT],
-                                               T (&red)[NWAVES / 2][16][TileCols<T, NG, LW>::CP], T *act,
+                                               T (&red)[NT][16][TileCols<T, NG, LW>::CP], T *act,
                                                long B, long M, long b0, long j0, long ncol,
                                                typename Real<T>::acc_t tail = {}) {
+  static_assert(NT == NWAVES / 2 || NT == NWAVES, "tiles of partial sums");
   using TC = TileCols<T, NG, LW>;
   constexpr int VW = Real<T>::VW;
   using vec_t = typename Real<T>::vec_t;
@@ -102,6 +106,27 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
   // the two); the row-wise epilogue then adds up the HALF published tiles.
   constexpr int HALF = NWAVES / 2;
   static_assert(NWAVES >= 2 && (NWAVES & (NWAVES - 1)) == 0, "a power of two, at least 2 wavefronts");
+  if constexpr (NT == NWAVES) {
+#pragma unroll
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        T *slot = &red[w][Real<T>::acc_row(q, v)][gcol(g, p)];
+        if (gwidth(g) == VW) {
+          vec_t t;
+#pragma unroll
+          for (int c = 0; c < VW; c++) t[c] = acc[g][c][v];
+          *reinterpret_cast<vec_t *>(slot) = t;
+        } else {
+#pragma unroll
+          for (int c = 0; c < LW; c++) slot[c] = acc[g][c][v];
+        }
+      }
+    if (TAIL && q == 0) {
+#pragma unroll
+      for (int v = 0; v < 4; v++) red[w][4 * (p >> 2) + v][tail_col0 + (p & 3)] = tail[v];
+    }
+  } else {
   if (w >= HALF) {
 #pragma unroll
     for (int g = 0; g < NG; g++)
@@ -145,6 +170,7 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
       for (int v = 0; v < 4; v++) red[w][4 * (p >> 2) + v][tail_col0 + (p & 3)] += tail[v];
     }
   }
+  }
   __syncthreads();
   // ---- bias (+ softmax): TPR threads per batch row, thread handles columns lr + TPR t
   constexpr int TPR = ForwardBias<T, NG, NWAVES>::TPR, PT = ForwardBias<T, NG, NWAVES>::PT;
@@ -156,7 +182,7 @@ __device__ __forceinline__ void forward_finish(const typename Real<T>::acc_t (&a
     const long col = lr + TPR * t;
     T sum = red[0][row][col < ncol ? col : 0];
 #pragma unroll
-    for (int h = 1; h < HALF; h++) sum += red[h][row][col < ncol ? col : 0];
+    for (int h = 1; h < NT; h++) sum += red[h][row][col < ncol ? col : 0];
     vals[t] = col < ncol ? sum + bv[t] : T(0);
     mx = (col < ncol && vals[t] > mx) ? vals[t] : mx;
   }
